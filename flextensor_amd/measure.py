@@ -1,0 +1,253 @@
+"""Build, check and time one candidate on the local GPU.
+
+Counterpart of the reference's flextensor/measure.py: ``build_and_eval``
+(:77-115) is tvm.build -> export_library -> load_module -> time_evaluator;
+here it is hiprtc -> hipModule -> hipEvent timing through libftrocm.so, with
+one step the reference lacks: before a timing is admitted the candidate's
+output is compared *on the device* with the output of the plain
+one-lane-per-output kernel of the same operator (templates/naive.hip), which
+plays the role of the reference's default-schedule build
+(flextensor/optimize/common.py:63-82). fp32 must satisfy
+max|out-ref| / max|ref| <= 1e-5; int32 must be identical.
+
+Candidates are evaluated in this process: forking a child per candidate, as
+the reference does (:55-74), is not safe once the HIP runtime is initialised.
+A failing candidate never propagates: callers map any exception to ``inf``.
+"""
+import ctypes
+import struct
+
+import numpy as np
+
+from . import runtime as rt
+from .plan import KernelPlan, current_stream
+from .templates import gfx950
+from .utils import to_tuple, ceil_div
+
+FP32_TOL = 1e-5
+# buffers of a memory-bound operator are rotated so that consecutive timed
+# launches do not find their data in the 256 MB last-level cache
+LLC_BYTES = 256 << 20
+MAX_SETS = 24
+
+
+class WrongResult(RuntimeError):
+    """A candidate kernel ran but its output failed the correctness gate."""
+
+
+def seeded_inputs(bufs, seed=0):
+    """Host arrays for the input buffers: fp32 uniform[-1,1), int8 uniform
+    over [-128,127], from numpy's default_rng(seed)."""
+    rng = np.random.default_rng(seed)
+    arrays = []
+    for b in bufs[:-1]:
+        shape = to_tuple(b.shape)
+        if b.dtype == "float32":
+            arrays.append(rng.uniform(-1.0, 1.0, size=shape).astype(np.float32))
+        elif b.dtype == "int8":
+            arrays.append(rng.integers(-128, 128, size=shape, dtype=np.int8))
+        else:
+            raise ValueError("no input generator for dtype %s" % b.dtype)
+    return arrays
+
+
+_naive_modules = {}
+
+
+def _naive(kernel):
+    if kernel not in _naive_modules:
+        src = gfx950.template_source("naive.hip")
+        _naive_modules[kernel] = rt.Module(rt.compile_to_code(src, []), kernel)
+    return _naive_modules[kernel]
+
+
+def _grid1d(n, cap=None):
+    g = ceil_div(int(n), 256)
+    if cap:
+        g = min(g, cap)
+    return (max(g, 1), 1, 1)
+
+
+def run_default_schedule(ops, tensors, stream=0):
+    """Run the task with the plain per-output kernels (the 'default schedule').
+
+    ``ops`` is the task's output op list; ``tensors`` are device tensors in
+    ``bufs`` order and the last one receives the result. Intermediate
+    operators (padding) are folded into the consumer's index predicate, which
+    is what the operator definitions compute.
+    """
+    op = ops[0]
+    i32 = ctypes.c_int
+    out = tensors[-1]
+    if op.kind == "gemm":
+        if op.attrs.get("transposeA"):
+            raise NotImplementedError("transposeA")
+        M, N = [a.extent for a in op.axis]
+        K = op.reduce_axis[0].extent
+        args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(out), i32(M), i32(N), i32(K),
+                i32(1 if op.attrs.get("transposeB") else 0)]
+        _naive("gemm_f32_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
+    elif op.kind == "gemm_int8":
+        M, N = [a.extent for a in op.axis]
+        K = op.reduce_axis[0].extent
+        args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(out), i32(M), i32(N), i32(K)]
+        _naive("gemm_i8_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
+    elif op.kind == "conv2d_nchw":
+        a = op.attrs
+        b, ko, p, q = [x.extent for x in op.axis]
+        _, c, h, w = a["in_shape"]
+        s, r = op.reduce_axis[1].extent, op.reduce_axis[2].extent
+        args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(out)] + [i32(v) for v in (
+            b, c, h, w, ko, r, s, a["stride"][0], a["stride"][1], a["padding"][0], a["padding"][1],
+            a["dilation"][0], a["dilation"][1], a["groups"], p, q)]
+        _naive("conv2d_nchw_naive").launch(_grid1d(b * ko * p * q), (256, 1, 1), args, stream=stream)
+    elif op.kind == "depthwise_conv2d_nchw":
+        a = op.attrs
+        b, co, p, q = [x.extent for x in op.axis]
+        _, c, h, w = a["in_shape"]
+        s, r = op.reduce_axis[0].extent, op.reduce_axis[1].extent
+        args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(out)] + [i32(v) for v in (
+            b, c, h, w, a["factor"], r, s, a["stride"][0], a["stride"][1], a["padding"][0],
+            a["padding"][1], a["dilation"][0], a["dilation"][1], p, q)]
+        _naive("depthwise_nchw_naive").launch(_grid1d(b * co * p * q), (256, 1, 1), args, stream=stream)
+    elif op.kind == "zero_pad2d":
+        b, c, ph, pw = [x.extent for x in op.axis]
+        pt, pb, pl, pr = op.attrs["padding"]
+        args = [rt.ptr(tensors[0]), rt.ptr(out)] + [i32(v) for v in (
+            b * c, ph - pt - pb, pw - pl - pr, pt, pb, pl, pr)]
+        _naive("zero_pad2d_naive").launch(_grid1d(b * c * ph * pw), (256, 1, 1), args, stream=stream)
+    else:
+        raise NotImplementedError("no default-schedule kernel for %s" % op.kind)
+
+
+def compare_on_device(out, ref, stream=0):
+    """(passed, metric) with metric = max|out-ref|/max|ref| for fp32 tensors and
+    the number of differing entries for int32 tensors."""
+    import torch
+    n = out.numel()
+    res = torch.zeros(2, dtype=torch.int32, device=out.device)
+    args = [rt.ptr(out), rt.ptr(ref), ctypes.c_longlong(n), rt.ptr(res)]
+    if out.dtype == torch.float32:
+        _naive("check_f32").launch(_grid1d(n, 2048), (256, 1, 1), args, stream=stream)
+        bits = res.cpu().numpy().astype(np.uint32)
+        md, mr = struct.unpack("ff", bits.tobytes())
+        if not np.isfinite(md):
+            return False, float("inf")
+        rel = md / mr if mr > 0 else md
+        return rel <= FP32_TOL, rel
+    if out.dtype == torch.int32:
+        _naive("check_i32").launch(_grid1d(n, 2048), (256, 1, 1), args, stream=stream)
+        bad = int(res.cpu().numpy().astype(np.uint32)[0])
+        return bad == 0, float(bad)
+    raise ValueError("no comparison for dtype %s" % out.dtype)
+
+
+class Measurer(object):
+    """Device-resident inputs and the default-schedule result of one task."""
+
+    def __init__(self, task_key, seed=0):
+        import torch
+        from .task import TASK_TABLE
+        if not torch.cuda.is_available():
+            raise rt.RuntimeError_("no GPU visible: candidates can only be measured on a device")
+        self.task_key = task_key
+        task = TASK_TABLE[task_key]
+        self.ops, self.bufs = task.func(*task.args)
+        torch.cuda.set_device(task.dev_id if task.dev_id < torch.cuda.device_count() else 0)
+        host = seeded_inputs(self.bufs, seed)
+        out_b = self.bufs[-1]
+        tdt = {"float32": torch.float32, "int32": torch.int32}[out_b.dtype]
+        bytes_per_set = sum(a.nbytes for a in host) + int(np.prod(out_b.shape)) * 4
+        kind = self.ops[0].kind
+        if kind == "depthwise_conv2d_nchw":
+            nsets = int(min(MAX_SETS, max(1, ceil_div(2 * LLC_BYTES, bytes_per_set))))
+        else:
+            nsets = 1
+        self.sets = []
+        for i in range(nsets):
+            ins = [torch.from_numpy(a).cuda() for a in host]
+            self.sets.append(ins + [torch.empty(to_tuple(out_b.shape), dtype=tdt, device="cuda")])
+        self.ref = torch.empty(to_tuple(out_b.shape), dtype=tdt, device="cuda")
+        run_default_schedule(self.ops, self.sets[0][:-1] + [self.ref], stream=current_stream())
+        torch.cuda.synchronize()
+
+    def check(self, out):
+        import torch
+        ok, metric = compare_on_device(out, self.ref, stream=current_stream())
+        torch.cuda.synchronize()
+        return ok, metric
+
+    def evaluate(self, plan, number=10, warmup=2):
+        """ms per run of ``plan``; raises on build failure or wrong output."""
+        import torch
+        built = plan.build()
+        try:
+            first = self.sets[0]
+            first[-1].zero_()
+            built(*first)
+            torch.cuda.synchronize()
+            ok, metric = self.check(first[-1])
+            if not ok:
+                raise WrongResult("output differs from the default schedule (metric %g)" % metric)
+            return built.time(self.sets, warmup=warmup, iters=max(int(number), 1))
+        finally:
+            built.close()
+
+
+_measurers = {}
+
+
+def get_measurer(task_key, seed=0):
+    key = (task_key, seed)
+    if key not in _measurers:
+        _measurers.clear()  # one task at a time keeps device memory bounded
+        _measurers[key] = Measurer(task_key, seed)
+    return _measurers[key]
+
+
+def build_and_eval(lib, s, bufs, target, dev_id, rpc_info=None, number=1):
+    """Build plan ``s``, verify it, time ``number`` launches; returns mean ms.
+
+    ``lib`` (a path the reference writes the exported library to) receives the
+    code object of the plan's last kernel when it is not None.
+    """
+    if not isinstance(s, KernelPlan):
+        raise TypeError("build_and_eval expects a KernelPlan")
+    if rpc_info is not None and getattr(rpc_info, "use_rpc", None):
+        raise RuntimeError("remote measurement is not supported by the gfx950 backend")
+    if lib:
+        codes = s.compile()
+        with open(lib, "wb") as f:
+            f.write(codes[-1])
+    return get_measurer(s.task_key).evaluate(s, number=number)
+
+
+def _evaluate(s, bufs, target, dev_id, number=1, q=None):
+    """In-process build + time (flextensor/measure.py:29-52)."""
+    time_cost = build_and_eval(None, s, bufs, target, dev_id, None, number)
+    if q:
+        q.put(time_cost)
+    return time_cost
+
+
+def servant_routine(func, que, *args, **kwargs):
+    try:
+        ret = func(*args, **kwargs)
+    except Exception as e:  # noqa: BLE001 - every failure becomes a value
+        ret = e
+    que.put(ret)
+
+
+def master_routine(timeout, func, *args, **kwargs):
+    """Run ``func`` and return its result, or the exception it raised.
+
+    The reference runs ``func`` in a forked child and waits ``timeout`` seconds
+    (flextensor/measure.py:63-74). A process that has initialised the GPU must
+    not fork, so the call is made in-process; kernels built from the templates
+    have compile-time loop bounds and always terminate.
+    """
+    del timeout
+    try:
+        return func(*args, **kwargs)
+    except Exception as e:  # noqa: BLE001
+        return e

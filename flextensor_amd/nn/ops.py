@@ -1,0 +1,137 @@
+"""Operator definitions: the numerics contract of the tuned kernels.
+
+Each function mirrors the signature and the index expression of its
+counterpart in the reference's flextensor/nn/ops.py and returns the output
+``Tensor`` of a ``ComputeOp`` that the gfx950 templates know how to lower.
+The CPU restatement of the same expressions lives in oracle/.
+"""
+from ..te import ComputeOp, IterVar
+
+
+def _pair(v, what):
+    if isinstance(v, int):
+        return (v, v)
+    v = tuple(int(x) for x in v)
+    if len(v) != 2:
+        raise ValueError("%s must be an int or a pair, got %r" % (what, v))
+    return v
+
+
+def zero_pad2d(inputs, padding=0):
+    """P[b,c,h,w] = X[b,c,h-pt,w-pl] inside the image, 0 outside.
+
+    Follows flextensor/nn/ops.py:83-117 (padding is an int, (ph, pw) or
+    (top, bottom, left, right)).
+    """
+    if isinstance(padding, int):
+        padding = (padding,) * 4
+    padding = tuple(int(p) for p in padding)
+    if len(padding) == 2:
+        padding = (padding[0], padding[0], padding[1], padding[1])
+    if len(padding) != 4:
+        raise ValueError("padding must have 1, 2 or 4 entries")
+    b, c, h, w = inputs.shape
+    out_shape = (b, c, h + padding[0] + padding[1], w + padding[2] + padding[3])
+    axis = [IterVar(n, e) for n, e in zip("bchw", out_shape)]
+    op = ComputeOp("Padding", "zero_pad2d", out_shape, inputs.dtype, axis, [], [inputs],
+                   {"padding": padding})
+    return op.output(0)
+
+
+def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
+    """O[b,k,h,w] = sum_{rc,rw,rh} P[b, (k//Kg)*Cg+rc, h*s+rh*d, w*s+rw*d] * W[k,rc,rh,rw].
+
+    Follows flextensor/nn/ops.py:419-479: the padded input is its own operator
+    (so the graph is [Padding, conv]); reduce axes are declared [rc, rw, rh];
+    out = (in + 2p - d(k-1) - 1)//s + 1.
+    """
+    if bias is not None:
+        raise NotImplementedError("bias epilogue is not part of the tuned path")
+    batch, in_c, in_h, in_w = inputs.shape
+    out_c, c_per_group, k_h, k_w = weight.shape
+    if c_per_group * groups != in_c:
+        raise ValueError("weight channels %d * groups %d != input channels %d"
+                         % (c_per_group, groups, in_c))
+    if out_c % groups != 0:
+        raise ValueError("output channels not divisible by groups")
+    stride = _pair(stride, "stride")
+    padding = _pair(padding, "padding")
+    dilation = _pair(dilation, "dilation")
+    out_h = (in_h + 2 * padding[0] - dilation[0] * (k_h - 1) - 1) // stride[0] + 1
+    out_w = (in_w + 2 * padding[1] - dilation[1] * (k_w - 1) - 1) // stride[1] + 1
+    padded = zero_pad2d(inputs, padding=padding)
+    out_shape = (batch, out_c, out_h, out_w)
+    axis = [IterVar(n, e) for n, e in zip("bchw", out_shape)]
+    raxis = [IterVar("rc", c_per_group, "reduce"), IterVar("rw", k_w, "reduce"),
+             IterVar("rh", k_h, "reduce")]
+    op = ComputeOp("compute", "conv2d_nchw", out_shape, inputs.dtype, axis, raxis,
+                   [padded, weight],
+                   {"stride": stride, "padding": padding, "dilation": dilation,
+                    "groups": int(groups), "in_shape": inputs.shape})
+    return op.output(0)
+
+
+def depthwise_conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1):
+    """O[b,c,h,w] = sum_{rw,rh} P[b, c//f, h*s+rh*d, w*s+rw*d] * W[c//f, c%f, rh, rw].
+
+    Follows flextensor/nn/ops.py:622-678; weight layout [C, factor, kh, kw].
+    """
+    if bias is not None:
+        raise NotImplementedError("bias epilogue is not part of the tuned path")
+    batch, in_c, in_h, in_w = inputs.shape
+    w_c, factor, k_h, k_w = weight.shape
+    if w_c != in_c:
+        raise ValueError("weight channels %d != input channels %d" % (w_c, in_c))
+    stride = _pair(stride, "stride")
+    padding = _pair(padding, "padding")
+    dilation = _pair(dilation, "dilation")
+    out_h = (in_h + 2 * padding[0] - dilation[0] * (k_h - 1) - 1) // stride[0] + 1
+    out_w = (in_w + 2 * padding[1] - dilation[1] * (k_w - 1) - 1) // stride[1] + 1
+    padded = zero_pad2d(inputs, padding=padding)
+    out_shape = (batch, in_c * factor, out_h, out_w)
+    axis = [IterVar(n, e) for n, e in zip("bchw", out_shape)]
+    raxis = [IterVar("rw", k_w, "reduce"), IterVar("rh", k_h, "reduce")]
+    op = ComputeOp("compute", "depthwise_conv2d_nchw", out_shape, inputs.dtype, axis, raxis,
+                   [padded, weight],
+                   {"stride": stride, "padding": padding, "dilation": dilation,
+                    "factor": int(factor), "in_shape": inputs.shape})
+    return op.output(0)
+
+
+def gemm(A, B, transposeA=False, transposeB=False):
+    """C[i,j] = sum_k A[i,k] * B[k,j] (operands optionally stored transposed).
+
+    Follows flextensor/nn/ops.py:1074-1108.
+    """
+    if transposeA:
+        k_a, m = A.shape
+    else:
+        m, k_a = A.shape
+    if transposeB:
+        n, k_b = B.shape
+    else:
+        k_b, n = B.shape
+    if k_a != k_b:
+        raise ValueError("reduce extents differ: %d vs %d" % (k_a, k_b))
+    axis = [IterVar("i", m), IterVar("j", n)]
+    raxis = [IterVar("k", k_a, "reduce")]
+    op = ComputeOp("compute", "gemm", (m, n), A.dtype, axis, raxis, [A, B],
+                   {"transposeA": bool(transposeA), "transposeB": bool(transposeB)})
+    return op.output(0)
+
+
+def gemm_int8(A, B):
+    """C[i,j] = sum_k int32(A[i,k]) * int32(B[j,k]); A [n,l], B [m,l] int8, C int32.
+
+    Follows flextensor/test/test_tvm/legacy/gemm_int8.py:15-21 (B is K-major).
+    """
+    if A.dtype != "int8" or B.dtype != "int8":
+        raise ValueError("gemm_int8 takes int8 operands")
+    m, k_a = A.shape
+    n, k_b = B.shape
+    if k_a != k_b:
+        raise ValueError("reduce extents differ: %d vs %d" % (k_a, k_b))
+    axis = [IterVar("i", m), IterVar("j", n)]
+    raxis = [IterVar("k", k_a, "reduce")]
+    op = ComputeOp("C", "gemm_int8", (m, n), "int32", axis, raxis, [A, B], {})
+    return op.output(0)

@@ -1,0 +1,129 @@
+"""Kernel plans: what ``schedule_with_config`` returns in place of a TVM schedule.
+
+A ``KernelPlan`` is the host-side description of how one task runs on the
+device: an ordered list of ``KernelSpec`` (template + constants + geometry)
+and the intermediate buffers between them. ``build`` compiles and loads the
+kernels and yields a callable over device tensors in ``bufs`` order — the
+counterpart of ``tvm.build(s, bufs, target)`` followed by ``func(*arrays)``
+in the reference (README.md:151-158, flextensor/optimize/common.py:34-48).
+"""
+import ctypes
+
+from . import runtime as rt
+
+
+class KernelPlan(object):
+    def __init__(self, task_key, bufs, specs, intermediates, configs):
+        self.task_key = task_key
+        self.bufs = list(bufs)
+        self.specs = list(specs)
+        # name -> (shape, dtype) of buffers the plan owns (e.g. a padded image)
+        self.intermediates = dict(intermediates)
+        self.configs = configs
+        # argument names of the caller's buffers, inputs..., output
+        self.buf_names = ["in%d" % i for i in range(len(bufs) - 1)] + ["out"]
+
+    def describe(self):
+        return [(s.kernel, dict(s.defines), s.grid, s.block) for s in self.specs]
+
+    def compile(self, arch=rt.DEFAULT_ARCH):
+        """Compile every kernel to a code object (no device needed)."""
+        return [rt.compile_to_code(s.source(), s.options(), arch) for s in self.specs]
+
+    def build(self):
+        return BuiltPlan(self)
+
+    def __repr__(self):
+        return "KernelPlan(%s: %s)" % (self.task_key, ", ".join(s.kernel for s in self.specs))
+
+
+_TORCH_DTYPES = None
+
+
+def _torch_dtype(name):
+    global _TORCH_DTYPES
+    import torch
+    if _TORCH_DTYPES is None:
+        _TORCH_DTYPES = {"float32": torch.float32, "int8": torch.int8, "int32": torch.int32}
+    return _TORCH_DTYPES[name]
+
+
+def current_stream():
+    """Handle of the stream device work is enqueued on (torch's current one)."""
+    import torch
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+class BuiltPlan(object):
+    """Loaded kernels of a plan; call it with device tensors in ``bufs`` order."""
+
+    def __init__(self, plan):
+        import torch
+        if not torch.cuda.is_available():
+            raise rt.RuntimeError_("no GPU visible: a kernel plan can only be built on a device")
+        self.plan = plan
+        self.modules = []
+        for spec, code in zip(plan.specs, plan.compile()):
+            self.modules.append(rt.Module(code, spec.kernel))
+        self.scratch = {}
+        for name, (shape, dtype) in plan.intermediates.items():
+            self.scratch[name] = torch.empty(shape, dtype=_torch_dtype(dtype), device="cuda")
+
+    def attrs(self):
+        return [m.attrs() for m in self.modules]
+
+    def _check(self, tensors):
+        plan = self.plan
+        if len(tensors) != len(plan.bufs):
+            raise ValueError("expected %d tensors (inputs..., output), got %d"
+                             % (len(plan.bufs), len(tensors)))
+        for t, b in zip(tensors, plan.bufs):
+            if tuple(t.shape) != tuple(b.shape):
+                raise ValueError("tensor shape %s does not match %s" % (tuple(t.shape), b))
+            if t.dtype != _torch_dtype(b.dtype):
+                raise ValueError("tensor dtype %s does not match %s" % (t.dtype, b))
+            if not t.is_cuda or not t.is_contiguous():
+                raise ValueError("tensors must be contiguous device tensors")
+
+    def launches(self, tensors):
+        """Launch descriptors of one run over ``tensors`` (validated)."""
+        self._check(tensors)
+        named = dict(zip(self.plan.buf_names, tensors))
+        named.update(self.scratch)
+        out = []
+        for spec, mod in zip(self.plan.specs, self.modules):
+            vals = []
+            for kind, v in spec.args:
+                if kind == "buf":
+                    vals.append(rt.ptr(named[v]))
+                elif kind == "i32":
+                    vals.append(ctypes.c_int(int(v)))
+                elif kind == "u32":
+                    vals.append(ctypes.c_uint(int(v)))
+                elif kind == "i64":
+                    vals.append(ctypes.c_longlong(int(v)))
+                else:
+                    raise ValueError("unknown argument kind %s" % kind)
+            out.append(rt.Launch(mod, spec.grid, spec.block, vals, spec.lds_bytes))
+        return out
+
+    def __call__(self, *tensors):
+        rt.launch_seq(self.launches(tensors), stream=current_stream())
+
+    def time(self, tensor_sets, warmup=2, iters=10):
+        """Mean ms per run, rotating through ``tensor_sets``."""
+        sets = [self.launches(ts) for ts in tensor_sets]
+        return rt.time_seq(sets, warmup=warmup, iters=iters, stream=current_stream())
+
+    def close(self):
+        for m in self.modules:
+            m.close()
+        self.modules = []
+
+
+def build(s, bufs=None, target=None):
+    """``build(s, bufs, target)``: the call a user of the reference makes with
+    ``tvm.build`` on the result of ``schedule`` / ``schedule_with_config``."""
+    if not isinstance(s, KernelPlan):
+        raise TypeError("expected the plan returned by schedule()/schedule_with_config()")
+    return s.build()

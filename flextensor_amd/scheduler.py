@@ -1,0 +1,659 @@
+"""Search driver and config replay.
+
+Keeps the reference's entry points and their signatures
+(flextensor/scheduler.py): ``schedule`` (:969-1111), ``schedule_with_config``
+(:1114-1130), ``schedule_with_config_ops`` (:1133-1186), ``Scheduler`` with
+``_warm_up`` (:222-280), ``_random_schedule`` (:282-291) and
+``_searching_schedule`` (:293-442), ``OpScheduler`` (:767-822),
+``GraphScheduler`` (:863-920), ``flatten_graph`` (:36-55).
+
+What differs underneath: a config is lowered to hand-written gfx950 kernels
+(templates/gfx950.py) instead of TVM schedule primitives; candidates are
+compiled by a pool of ``parallel`` host workers (hiprtc, no device) and then
+checked and timed one at a time on the GPU in this process (measure.py).
+"""
+import math
+import multiprocessing as mp
+import time
+from collections import deque
+from concurrent.futures import ProcessPoolExecutor
+
+import numpy as np
+
+from .model import WalkerGroup
+from .plan import KernelPlan
+from .space import Space, generate_space_inter_op, generate_space_intra_op
+from .task import TASK_TABLE
+from .te import ComputeOp
+from .templates import gfx950
+from .utils import Config, assert_print
+
+SUPPORTED_TARGETS = ("rocm",)
+
+
+def flatten_graph(ops):
+    """Compute ops in producer->consumer order plus tensor -> consumers map."""
+    bfs_order = []
+    down_graph = {}
+    visited = set()
+    q = deque()
+    for op in ops:
+        q.append(op)
+        visited.add(op)
+    while q:
+        cur = q.popleft()
+        if isinstance(cur, ComputeOp):
+            bfs_order.append(cur)
+        for t in cur.input_tensors:
+            if t.op not in visited:
+                visited.add(t.op)
+                q.append(t.op)
+            down_graph.setdefault(t, []).append(cur)
+    return list(reversed(bfs_order)), down_graph
+
+
+class OpState(object):
+    def __init__(self):
+        self.inline = False
+        self.loop_lst = []
+        self.loop_idx = []
+        self.compute_at = False
+        self.consumer_lst = []
+
+
+def _empty_config():
+    return {k: [] for k in Space.valid_type_keys}
+
+
+# --------------------------------------------------------------------------
+# parallel compilation of candidates (host only)
+# --------------------------------------------------------------------------
+
+def _compile_job(template, options, arch):
+    """Worker: compile one kernel into the on-disk cache. Returns an error
+    string or None. Runs in a spawned process that never touches the GPU."""
+    try:
+        from . import runtime as rt
+        rt.compile_to_code(gfx950.template_source(template), options, arch)
+        return None
+    except Exception as e:  # noqa: BLE001
+        return str(e)
+
+
+class CompilePool(object):
+    def __init__(self, workers):
+        self.workers = max(int(workers), 1)
+        self._pool = None
+
+    def _ensure(self):
+        if self._pool is None and self.workers > 1:
+            self._pool = ProcessPoolExecutor(max_workers=self.workers,
+                                             mp_context=mp.get_context("spawn"))
+
+    def compile_plans(self, plans, timeout):
+        """Compile all kernels of ``plans`` (None entries skipped). Returns one
+        error string or None per plan."""
+        from . import runtime as rt
+        errors = [None] * len(plans)
+        jobs = {}
+        for i, plan in enumerate(plans):
+            if plan is None:
+                continue
+            for spec in plan.specs:
+                key = (spec.template, tuple(spec.options()))
+                jobs.setdefault(key, []).append(i)
+        if not jobs:
+            return errors
+        self._ensure()
+        if self._pool is None:
+            for key, owners in jobs.items():
+                err = _compile_job(key[0], list(key[1]), rt.DEFAULT_ARCH)
+                if err:
+                    for i in owners:
+                        errors[i] = err
+            return errors
+        futs = {}
+        try:
+            for key in jobs:
+                futs[key] = self._pool.submit(_compile_job, key[0], list(key[1]), rt.DEFAULT_ARCH)
+            deadline = time.time() + max(float(timeout), 1.0) * max(1, math.ceil(len(jobs) / self.workers))
+            for key, fut in futs.items():
+                try:
+                    err = fut.result(timeout=max(deadline - time.time(), 0.5))
+                except Exception as e:  # noqa: BLE001  (timeout or broken pool)
+                    err = "compile failed: %r" % (e,)
+                    if not fut.done():
+                        self.close(kill=True)
+                if err:
+                    for i in jobs[key]:
+                        errors[i] = err
+        except Exception as e:  # noqa: BLE001
+            self.close(kill=True)
+            for key, owners in jobs.items():
+                for i in owners:
+                    errors[i] = errors[i] or "compile pool failed: %r" % (e,)
+        return errors
+
+    def close(self, kill=False):
+        if self._pool is not None:
+            try:
+                if kill:
+                    for p in list(getattr(self._pool, "_processes", {}).values()):
+                        p.terminate()
+                self._pool.shutdown(wait=not kill, cancel_futures=True)
+            except Exception:  # noqa: BLE001
+                pass
+            self._pool = None
+
+
+def build_and_eval_wrapper(lib, task_key, config, op_pos=None, rpc_info=None, rewrite=False,
+                           number=1):
+    from .measure import build_and_eval
+    task = TASK_TABLE[task_key]
+    s, bufs = schedule_with_config(task_key, config, op_pos=op_pos, rewrite=rewrite)
+    return build_and_eval(lib, s, bufs, task.target, task.dev_id, rpc_info, number)
+
+
+class Scheduler(object):
+    def __init__(self, name, task_key, space, parallel=2, timeout=4.0, trial=100, number=1,
+                 early_stop=30, rpc_info=None, rewrite=False, evaluator=None):
+        self.task_key = task_key
+        self.space = space
+        self.parallel = max(parallel, 1)
+        self.timeout = timeout
+        self.trial = trial
+        self.number = number
+        self.early_stop = early_stop
+        self.task = TASK_TABLE[self.task_key]
+        self.walker_group = WalkerGroup(self.task.category + "_" + name, self.space)
+        self.rpc_info = rpc_info
+        self.rewrite = rewrite
+        # evaluator(task_key, Config, op_pos, number) -> ms; None = measure on the GPU
+        self.evaluator = evaluator
+
+        self.re_evalutate_number = 10
+        self.warm_up_epoch = 20
+        self.warm_up_number = 20
+        self.verbose = True
+        self._pool = None
+        self.op_pos = None
+
+    def _log(self, *args):
+        if self.verbose:
+            print(*args, flush=True)
+
+    # ---- warm-up: random points ---------------------------------------
+    def _warm_up(self, warm_up_epoches, warm_up_trials, configs, type_keys, max_repeat=20,
+                 use_model=False):
+        warm_up_enough = False
+        count_repeat = 0
+        old_timeout = self.timeout
+        while not warm_up_enough:
+            for ep in range(warm_up_epoches):
+                warm_up_ret = self.walker_group.forward(warm_up_trials, policy="random")
+                warm_up_configs = [{} for _ in range(warm_up_trials)]
+                warm_up_indices = [{} for _ in range(warm_up_trials)]
+                for count in range(warm_up_trials):
+                    config = warm_up_configs[count]
+                    for type_key in type_keys:
+                        config[type_key] = []
+                        for name in self.space.types[type_key]:
+                            entity = warm_up_ret[name][0][count]
+                            warm_up_indices[count][name] = int(warm_up_ret[name][1][count])
+                            config[type_key].append(entity)
+                # points already measured are not measured again
+                fresh = [i for i in range(warm_up_trials)
+                         if not self.walker_group.ever_met(warm_up_indices[i])]
+                seen = set()
+                uniq = []
+                for i in fresh:
+                    k = str(warm_up_indices[i])
+                    if k not in seen:
+                        seen.add(k)
+                        uniq.append(i)
+                results = self.parallel_evaluate(configs, [warm_up_configs[i] for i in uniq],
+                                                 number=self.number)
+                self.walker_group.add_perf_data([warm_up_indices[i] for i in uniq], results)
+                self._log("warm up [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+                for i, res in zip(uniq, results):
+                    if res < float("inf"):
+                        self.walker_group.record(warm_up_indices[i], res)
+                    else:
+                        self.walker_group.visit.add(str(warm_up_indices[i]))
+            if not self.walker_group.top1():
+                self._log("Warning: No valid schedule found in warm up process, please use more trials")
+                self._log("Now automatically use more trials, increase %d" % warm_up_trials)
+                warm_up_epoches = 1
+                count_repeat += 1
+                self.timeout = min(2 * self.timeout, 40)
+                if count_repeat >= max_repeat:
+                    self._log("Fail to find valid schedule, too many errors")
+                    warm_up_enough = True
+            else:
+                warm_up_enough = True
+        self.timeout = old_timeout
+
+    def _seed(self, configs, type_keys):
+        """Measure the template's default config first (when it is a point of
+        the space) so that the walk has a sane starting point."""
+        if self.op_pos is None:
+            return
+        ops, _ = self.task.func(*self.task.args)
+        op = flatten_graph(ops)[0][self.op_pos]
+        try:
+            cfg = gfx950.default_config(op)
+        except Exception:  # noqa: BLE001
+            return
+        indices = {}
+        for type_key in type_keys:
+            names = self.space.types[type_key]
+            ents = cfg.get(type_key, [])
+            if len(names) != len(ents):
+                return
+            for name, ent in zip(names, ents):
+                try:
+                    indices[name] = self.space.subspaces[name].static_entities.index(list(ent))
+                except ValueError:
+                    return
+        if self.walker_group.ever_met(indices):
+            return
+        res = self.parallel_evaluate(configs, [self.walker_group.to_config(indices)],
+                                     number=self.number)
+        self._log("seed [%.6f] [ %.6f ]" % (time.time(), res[0]))
+        if res[0] < float("inf"):
+            self.walker_group.record(indices, res[0])
+        else:
+            self.walker_group.visit.add(str(indices))
+
+    def _random_schedule(self, configs, type_keys, use_model=False):
+        for trial in range(self.trial):
+            self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+        return self.walker_group.to_config(self.walker_group.top1())
+
+    # ---- neighbourhood search -----------------------------------------
+    def _searching_schedule(self, configs, type_keys, use_model=False):
+        self._seed(configs, type_keys)
+        self._warm_up(self.warm_up_epoch, self.warm_up_number, configs, type_keys,
+                      use_model=use_model)
+
+        minimal = [{}, float("inf")]
+        retired_indices = []
+
+        part = math.ceil(self.trial / 20)
+        value_early_stop = self.walker_group.top1_value()
+        early_stop_count = 0
+        count_incessant_empty_trial = 0
+        for trial in range(self.trial):
+            if not self.walker_group.has_more():
+                self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+                continue
+            from_indices, from_value = self.walker_group.top_random(with_value=True)
+            next_indices_lst, action_lst = self.walker_group.full_walk(from_indices, no_repeat=True)
+            next_configs = [self.walker_group.to_config(indices) for indices in next_indices_lst]
+            if len(next_configs) < 1:
+                count_incessant_empty_trial += 1
+            else:
+                count_incessant_empty_trial = 0
+            results = self.parallel_evaluate(configs, next_configs, number=self.number)
+            self.walker_group.add_perf_data(next_indices_lst, results)
+            self._log("tune [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+            rewards = [np.tanh(max(from_value - result, 0.0)) for result in results]
+
+            is_local_minimal = True
+            for indices, action, reward, result in zip(next_indices_lst, action_lst, rewards, results):
+                self.walker_group.add_data(action[0], from_indices, action[1], indices, reward)
+                self.walker_group.record(indices, result, random_reject=True)
+                if result < self.walker_group.top1_value():
+                    is_local_minimal = False
+            if is_local_minimal or count_incessant_empty_trial > 0:
+                top = self.walker_group.pop_top()
+                if top.value < minimal[1]:
+                    if minimal[1] < float("inf"):
+                        retired_indices.append(minimal)
+                    minimal = [top.indices, top.value]
+                else:
+                    retired_indices.append([top.indices, top.value])
+            if self.walker_group.top1_value() < minimal[1]:
+                cur_best_value = self.walker_group.top1_value()
+                cur_best = self.walker_group.top1()
+            else:
+                cur_best_value = minimal[1]
+                cur_best = minimal[0]
+            self._log("No. %d | [%.6f] The best currently %.6f" % (trial, time.time(), cur_best_value),
+                      cur_best)
+            if count_incessant_empty_trial >= self.early_stop:
+                self._log("Early stop after continuous no trials %d times" % count_incessant_empty_trial)
+                break
+            # "no progress" = the best moved by less than 2 % (the reference uses
+            # an absolute 0.02 ms, which every microsecond-scale kernel satisfies)
+            if value_early_stop < float("inf") and \
+                    math.fabs(cur_best_value - value_early_stop) < 0.02 * value_early_stop:
+                early_stop_count += 1
+            else:
+                value_early_stop = cur_best_value
+                early_stop_count = 0
+            if early_stop_count >= self.early_stop:
+                self._log("Early stop with value %f repeats %d times" % (value_early_stop, early_stop_count))
+                break
+            if (trial + 1) % part == 0:
+                # re-measure the current top points one after another
+                if minimal[1] < float("inf"):
+                    self.walker_group.record(minimal[0], minimal[1], random_reject=False)
+                for retired in retired_indices:
+                    self.walker_group.record(retired[0], retired[1], random_reject=False)
+                retired_indices = []
+                minimal = [{}, float("inf")]
+                indices_lst = self.walker_group.topk(self.re_evalutate_number, modify=True)
+                next_configs = [self.walker_group.to_config(indices) for indices in indices_lst]
+                results = self.parallel_evaluate(configs, next_configs, number=self.number)
+                self.walker_group.add_perf_data(indices_lst, results)
+                self._log("re-evaluate [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+                for indices, result in zip(indices_lst, results):
+                    if result < float("inf"):
+                        self.walker_group.record(indices, result, random_reject=False)
+                self.walker_group.clear_data()
+            self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+        if self.walker_group.top1_value() < minimal[1]:
+            best = self.walker_group.top1()
+        else:
+            best = minimal[0]
+        return self.walker_group.to_config(best)
+
+    # ---- evaluation ----------------------------------------------------
+    def _fetch_config(self, old_configs, config, mode):
+        if mode == "op":
+            return Config(old_configs.op_config_lst + [config], old_configs.graph_config), self.op_pos
+        if mode == "graph":
+            return Config(old_configs.op_config_lst, config), None
+        raise RuntimeError("Unknown mode %s" % mode)
+
+    def _parallel_evaluate(self, old_configs, new_configs, mode="op", number=1):
+        """One cost in ms per new config; any failure is ``inf``."""
+        if not new_configs:
+            return []
+        built = [self._fetch_config(old_configs, c, mode) for c in new_configs]
+        if self.evaluator is not None:
+            res = []
+            for cfg, op_pos in built:
+                try:
+                    res.append(float(self.evaluator(self.task_key, cfg, op_pos, number)))
+                except Exception:  # noqa: BLE001
+                    res.append(float("inf"))
+            return res
+        from .measure import get_measurer
+        plans = []
+        for cfg, op_pos in built:
+            try:
+                s, _ = schedule_with_config(self.task_key, cfg, op_pos=op_pos, rewrite=self.rewrite)
+                plans.append(s)
+            except Exception:  # noqa: BLE001
+                plans.append(None)
+        if self._pool is None or self._pool.workers != self.parallel:
+            if self._pool is not None:
+                self._pool.close()
+            self._pool = CompilePool(self.parallel)
+        errors = self._pool.compile_plans(plans, self.timeout)
+        res = []
+        measurer = None
+        for plan, err in zip(plans, errors):
+            if plan is None or err is not None:
+                res.append(float("inf"))
+                continue
+            try:
+                if measurer is None:
+                    measurer = get_measurer(self.task_key)
+                res.append(float(measurer.evaluate(plan, number=number)))
+            except Exception:  # noqa: BLE001
+                res.append(float("inf"))
+        return res
+
+    def close(self):
+        if self._pool is not None:
+            self._pool.close()
+            self._pool = None
+
+
+class OpScheduler(Scheduler):
+    def __init__(self, task_key, op_pos, space, decay=0.7, parallel=1, timeout=4.0, trial=100,
+                 number=1, early_stop=30, rpc_info=None, rewrite=False, evaluator=None):
+        super(OpScheduler, self).__init__("op" + str(op_pos), task_key, space, parallel, timeout,
+                                          trial, number, early_stop, rpc_info, rewrite=rewrite,
+                                          evaluator=evaluator)
+        self.op_pos = op_pos
+
+    def schedule(self, configs, method="searching", use_model=False, perf_path=None):
+        wanted_types = ["fuse", "reorder", "spatial", "reduce", "unroll"]
+        if use_model:
+            raise RuntimeError("Currently no support for learned performance models")
+        if method == "searching":
+            return self._searching_schedule(configs, wanted_types, use_model=use_model)
+        elif method == "random":
+            return self._random_schedule(configs, wanted_types, use_model=use_model)
+        else:
+            raise RuntimeError("Currently no support for method %s" % method)
+
+    def parallel_evaluate(self, configs, next_op_configs, number=1, rpc_info=None):
+        return self._parallel_evaluate(configs, next_op_configs, mode="op", number=number)
+
+    @staticmethod
+    def generate_op_schedule(target, config):
+        """Return ``template(op, special, out_name, in_names, materialized_pad)``
+        -> list of KernelSpec for this target."""
+        if target == "rocm":
+            def template(op, special, out_name, in_names, materialized_pad=False):
+                return gfx950.lower(op, config, special, out_name, in_names, materialized_pad)
+            return template
+        raise RuntimeError("Currently no support for target %s" % target)
+
+
+class GraphScheduler(Scheduler):
+    def __init__(self, task_key, space, decay=0.7, parallel=10, timeout=4.0, trial=100, number=1,
+                 early_stop=30, rpc_info=None, rewrite=False, evaluator=None):
+        super(GraphScheduler, self).__init__("graph", task_key, space, parallel, timeout, trial,
+                                             number, early_stop, rpc_info, rewrite=rewrite,
+                                             evaluator=evaluator)
+
+    def schedule(self, configs, method="searching", use_model=False, perf_path=None):
+        types = ["inline", "merge", "special"]
+        if use_model:
+            raise RuntimeError("Currently no support for learned performance models")
+        if method == "searching":
+            return self._searching_schedule(configs, types, use_model=use_model)
+        elif method == "random":
+            return self._random_schedule(configs, types, use_model=use_model)
+        else:
+            raise RuntimeError("Currently no support for method %s" % method)
+
+    def parallel_evaluate(self, configs, graph_configs, number=1):
+        return self._parallel_evaluate(configs, graph_configs, mode="graph", number=number)
+
+
+# --------------------------------------------------------------------------
+# entry points
+# --------------------------------------------------------------------------
+
+def _op_states(op_lst, down_graph):
+    states = [OpState() for _ in op_lst]
+    for i, op in enumerate(op_lst):
+        consumers = []
+        for k in range(op.num_outputs):
+            if op.output(k) in down_graph:
+                consumers.extend(down_graph[op.output(k)])
+        states[i].consumer_lst = list(set(consumers))
+    return states
+
+
+def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=15, graph_stop=5,
+             number=1, timeout=5, parallel=8, method="searching", **kwargs):
+    """Tune a registered task; returns ``(s, bufs, configs)``.
+
+    Keyword extras understood (flextensor/scheduler.py:990-1014): ``trials``
+    (per-op trial counts), ``force_inline``, ``rpc_info`` (must not request a
+    remote session), ``use_model`` (must be false). Additional: ``evaluator``
+    (a cost function used instead of the GPU, for host-only tests),
+    ``warm_up`` = (epochs, points per epoch), ``verbose``.
+    """
+    task = TASK_TABLE[task_key]
+    if task.target not in SUPPORTED_TARGETS:
+        raise RuntimeError("Currently no support for target %s" % task.target)
+    if method not in ("searching", "random"):
+        raise RuntimeError("Currently no support for method %s" % method)
+    ops, bufs = task.func(*task.args)
+    op_lst, down_graph = flatten_graph(ops)
+    _op_states(op_lst, down_graph)
+
+    if "trials" in kwargs:
+        assert_print(len(kwargs["trials"]) == len(op_lst), str(len(op_lst)))
+        force_trials = kwargs["trials"]
+    else:
+        force_trials = [op_trial for _ in op_lst]
+    if kwargs.get("use_model"):
+        raise RuntimeError("Currently no support for learned performance models")
+    force_inline = bool(kwargs.get("force_inline", False))
+    rpc_info = kwargs.get("rpc_info")
+    if rpc_info is not None and getattr(rpc_info, "use_rpc", None):
+        raise RuntimeError("remote measurement is not supported by the gfx950 backend")
+    evaluator = kwargs.get("evaluator")
+    warm_up = kwargs.get("warm_up")
+    verbose = kwargs.get("verbose", True)
+
+    graph_space = generate_space_inter_op(op_lst, down_graph, force_inline=force_inline,
+                                          special_space=task.special_space)
+    if verbose:
+        print("graph space size", len(graph_space))
+    total_size = len(graph_space)
+
+    if force_inline:
+        configs = Config([], {"inline": [graph_space.subspaces["inline"].static_entities[0]]})
+    else:
+        configs = Config([], None)
+
+    schedulers = []
+    try:
+        for pos, op in enumerate(op_lst):
+            space = generate_space_intra_op(op, down_graph, slevel=slevel, rlevel=rlevel,
+                                            target=task.target)
+            total_size *= max(len(space), 1)
+            if verbose:
+                print("op", pos, "space size:", len(space))
+            if len(space.subspaces) == 0 or \
+                    (force_inline and graph_space.subspaces["inline"].able_inline(pos)):
+                # nothing to decide for this op (e.g. padding, which has no knobs)
+                configs.op_config_lst.append(_empty_config() if len(space.subspaces) == 0 else {})
+                continue
+            op_scheduler = OpScheduler(task_key, pos, space, parallel=parallel, timeout=timeout,
+                                       trial=force_trials[pos], number=number, early_stop=op_stop,
+                                       rpc_info=rpc_info, evaluator=evaluator)
+            op_scheduler.verbose = verbose
+            if warm_up:
+                op_scheduler.warm_up_epoch, op_scheduler.warm_up_number = warm_up
+            schedulers.append(op_scheduler)
+            op_config = op_scheduler.schedule(configs, method=method)
+            configs.op_config_lst.append(op_config)
+
+        if verbose:
+            print("space size", total_size)
+
+        graph_scheduler = GraphScheduler(task_key, graph_space, parallel=parallel, timeout=timeout,
+                                         trial=graph_trial, number=number, early_stop=graph_stop,
+                                         rpc_info=rpc_info, evaluator=evaluator)
+        graph_scheduler.verbose = verbose
+        if warm_up:
+            graph_scheduler.warm_up_epoch, graph_scheduler.warm_up_number = warm_up
+        else:
+            # the graph space is tiny (inline flags x a few enumerated knobs)
+            graph_scheduler.warm_up_epoch = 2
+            graph_scheduler.warm_up_number = min(20, max(len(graph_space), 1))
+        schedulers.append(graph_scheduler)
+        graph_config = graph_scheduler.schedule(configs, method=method)
+        configs = Config(configs.op_config_lst, graph_config)
+    finally:
+        for sch in schedulers:
+            sch.close()
+
+    s, bufs = schedule_with_config(task_key, configs)
+    return s, bufs, configs
+
+
+def schedule_with_config(task_key, configs, op_pos=None, rewrite=False):
+    """Replay ``configs`` for a registered task; returns ``(s, bufs)`` where
+    ``s`` is a KernelPlan (``s.build()`` gives the callable)."""
+    task = TASK_TABLE[task_key]
+    if rewrite:
+        raise RuntimeError("the NCHWc rewrite is a CPU-only path of the reference")
+    if task.target not in SUPPORTED_TARGETS:
+        raise RuntimeError("Currently no support for target %s" % task.target)
+    ops, bufs = task.func(*task.args)
+    s, bufs = schedule_with_config_ops(ops, bufs, configs, op_pos=op_pos, target=task.target,
+                                       task_key=task_key, special_names=list(task.special_space))
+    return s, bufs
+
+
+def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", task_key=None,
+                             special_names=None):
+    """Lower an operator graph with given configs to a KernelPlan."""
+    if target not in SUPPORTED_TARGETS:
+        raise RuntimeError("Currently no support for target %s" % target)
+    if not isinstance(configs, Config):
+        configs = Config(configs[0], configs[1])
+    op_lst, down_graph = flatten_graph(ops)
+    op_states = _op_states(op_lst, down_graph)
+    op_config_lst = list(configs.op_config_lst)
+    if op_pos is not None:
+        assert_print(isinstance(op_pos, int), "op_pos should be int")
+        assert_print(op_pos < len(op_lst) and op_pos < len(op_config_lst), "op_pos too big")
+    else:
+        assert_print(len(op_config_lst) <= len(op_lst), "config length exceed op_lst")
+
+    # ---- graph level: which ops are folded into their consumer ----------
+    graph_config = configs.graph_config
+    inline_flags = None
+    if graph_config is not None and graph_config.get("inline"):
+        inline_flags = list(graph_config["inline"][0])
+    from .space import able_inline
+    for i, op in enumerate(op_lst):
+        if inline_flags is not None:
+            op_states[i].inline = bool(inline_flags[i]) if i < len(inline_flags) else False
+        else:
+            op_states[i].inline = able_inline(op, down_graph)  # default: fold padding in
+        if op_states[i].inline and not able_inline(op, down_graph):
+            raise gfx950.InvalidConfig("op %d cannot be inlined" % i)
+    special = None
+    if graph_config is not None and graph_config.get("special") and special_names:
+        special = dict(zip(special_names, graph_config["special"]))
+
+    # ---- name the buffers ------------------------------------------------
+    names = {}
+    for i, t in enumerate(bufs[:-1]):
+        names[t] = "in%d" % i
+    names[bufs[-1]] = "out"
+    intermediates = {}
+    specs = []
+    for i, op in enumerate(op_lst):
+        if op_states[i].inline:
+            continue
+        out_t = op.output(0)
+        if out_t not in names:
+            names[out_t] = "tmp%d" % i
+            intermediates[names[out_t]] = (out_t.shape, out_t.dtype)
+        in_names = []
+        materialized_pad = False
+        for t in op.input_tensors:
+            src = t
+            # an inlined producer is read through: the consumer sees its input
+            while isinstance(src.op, ComputeOp) and op_states[op_lst.index(src.op)].inline:
+                src = src.op.input_tensors[0]
+            if isinstance(t.op, ComputeOp) and t.op.kind == "zero_pad2d" and src is t:
+                materialized_pad = True
+            in_names.append(names[src])
+        config = op_config_lst[i] if i < len(op_config_lst) and op_config_lst[i] else None
+        if config is None or not any(config.get(k) for k in ("spatial", "reduce", "fuse")):
+            config = gfx950.default_config(op)
+        template = OpScheduler.generate_op_schedule(target, config)
+        specs.extend(template(op, special, names[out_t], in_names, materialized_pad))
+    return KernelPlan(task_key, bufs, specs, intermediates, configs), bufs
+
+
+def schedule_ops_with_config(s, op_lst, configs, target):
+    raise RuntimeError("schedule_ops_with_config operates on TVM schedules; "
+                       "use schedule_with_config_ops")

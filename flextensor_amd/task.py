@@ -1,0 +1,127 @@
+"""Tasks: named, registered operator instances to tune.
+
+Same contract as the reference's flextensor/task.py:29-57: ``Task`` builds
+its key as ``"{category}_{name}_{args}_{target}({dev_id})"``, keeps
+``func(*args) -> (ops, bufs)`` with bufs ordered inputs..., output, and can
+carry enumerated "special" knobs; ``register_task`` fills ``TASK_TABLE``.
+Drivers create a ``func=None`` task only to compute a key and then look the
+real one up (flextensor/optimize/optimize_gemm.py:26-35), so every shape that
+should be tunable is registered at import time, here for target ``"rocm"``.
+"""
+from .nn import conv2d_nchw, depthwise_conv2d_nchw, gemm as op_gemm, gemm_int8 as op_gemm_int8
+from .space import EnumSpace
+from .te import placeholder
+from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8,
+                             depthwise_shapes, baseline_conv_shapes, baseline_depthwise_shapes,
+                             baseline_gemm_shapes, baseline_gemm_int8_shapes)
+
+TASK_TABLE = {}
+
+ROCM_TARGET = "rocm"
+
+
+class Task(object):
+    def __init__(self, category, name, func, args, target, dev_id=0):
+        self.key = "{}_{}_{}_{}({})".format(category, name, args, target, dev_id)
+        self.func = func
+        self.args = args
+        self.target = target
+        self.dev_id = dev_id
+        self.category = category
+        self.special_space = {}
+
+    def set_specific_space(self, key, type, knobs):
+        if type == "enum":
+            self.special_space[key] = EnumSpace(knobs)
+        else:
+            raise RuntimeError("Not supported space type: %s" % type)
+
+
+def register_task(task, override=False):
+    if task.key in TASK_TABLE and not override:
+        return
+    TASK_TABLE[task.key] = task
+
+
+def register(func, category, name, args, target, dev_id=0, override=False):
+    task = Task(category, name, func, args, target, dev_id)
+    _attach_default_knobs(task)
+    register_task(task, override=override)
+
+
+# ---- operator wrappers: shapes -> (ops, bufs) ------------------------------
+
+def conv2d(N, C, H, W, K, kernel_size, stride=1, padding=0, dilation=1, groups=1):
+    """flextensor/task.py:74-78; bufs = [Img, W, Output], fp32, no bias."""
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((K, C // groups, kernel_size, kernel_size), name="W")
+    Output = conv2d_nchw(Img, Wt, stride=stride, padding=padding, dilation=dilation, groups=groups)
+    return [Output.op], [Img, Wt, Output]
+
+
+def depthwise_conv2d(N, C, H, W, factor, kernel_size, stride=1, padding=0, dilation=1):
+    """flextensor/task.py:96-100; weight [C, factor, k, k]."""
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((C, factor, kernel_size, kernel_size), name="W")
+    Output = depthwise_conv2d_nchw(Img, Wt, stride=stride, padding=padding, dilation=dilation)
+    return [Output.op], [Img, Wt, Output]
+
+
+def gemm(N, K, M):
+    """flextensor/task.py:145-149; A [N,K] · B [K,M] -> [N,M], fp32."""
+    A = placeholder((N, K), name="A")
+    B = placeholder((K, M), name="B")
+    Output = op_gemm(A, B)
+    return [Output.op], [A, B, Output]
+
+
+def gemm_int8(N, K, M):
+    """int8 A [N,K], int8 B [M,K] (K-major) -> int32 [N,M]
+    (flextensor/test/test_tvm/legacy/gemm_int8.py:15-21)."""
+    A = placeholder((N, K), dtype="int8", name="A")
+    B = placeholder((M, K), dtype="int8", name="B")
+    Output = op_gemm_int8(A, B)
+    return [Output.op], [A, B, Output]
+
+
+def _attach_default_knobs(task):
+    """Give a rocm task the enumerated knobs of its operator family."""
+    if task.target != ROCM_TARGET or task.func is None:
+        return
+    from .templates.gfx950 import special_knobs
+    kind = {gemm: "gemm", gemm_int8: "gemm_int8", conv2d: "conv2d_nchw",
+            depthwise_conv2d: "depthwise_conv2d_nchw"}.get(task.func)
+    if kind is None:
+        return
+    for key, knobs in special_knobs(kind).items():
+        if key not in task.special_space:
+            task.set_specific_space(key, "enum", knobs)
+
+
+# ---- registration ----------------------------------------------------------
+
+NUM_DEVICES = 4  # the reference registers every task for dev_id 0..3
+
+
+def _register_all():
+    for j in range(NUM_DEVICES):
+        for shape in gemm_shapes + baseline_gemm_shapes:
+            N, K, M = shape
+            register(gemm, "gemm", "gemm", (N, K, M), ROCM_TARGET, j)
+        for shape in baseline_gemm_int8_shapes:
+            N, K, M = shape
+            register(gemm_int8, "gemm", "gemm_int8", (N, K, M), ROCM_TARGET, j)
+        for name, shapes in (("yolo", yolo_shapes), ("yolo_b8", yolo_shapes_b8),
+                             ("baseline", baseline_conv_shapes)):
+            for i, shape in enumerate(shapes):
+                batch, in_c, h, w, out_c, _, k_h, k_w, _, stride, pad, dil, groups = shape
+                register(conv2d, "conv2d", name + str(i),
+                         (batch, in_c, h, w, out_c, k_h, stride, pad, dil, groups),
+                         ROCM_TARGET, j)
+        for shape in depthwise_shapes + baseline_depthwise_shapes:
+            batch, in_c, h, w, factor, k_h, k_w, stride, pad, dil = shape
+            register(depthwise_conv2d, "conv2d", "depthwise",
+                     (batch, in_c, h, w, factor, k_h, stride, pad, dil), ROCM_TARGET, j)
+
+
+_register_all()

@@ -1,0 +1,137 @@
+// Direct depthwise conv2d NCHW fp32 kernel template for gfx950, hiprtc-compiled.
+//
+//   O[b][c][h][w] = sum_{r,s} P[b][c / FACT][h*STR + r*DIL][w*STR + s*DIL]
+//                             * Wt[c / FACT][c % FACT][r][s]
+// with P the zero-padded input (padding folded into load predicates), as in
+// flextensor/nn/ops.py:622-678 (weight layout [C][FACT][R][S], ops.py:630).
+//
+// The operator moves ~2 bytes per flop: it is bound by HBM bandwidth, not by
+// arithmetic, so there is no matrix-core path. Each lane owns a TH x TW patch
+// of one output plane; consecutive lanes own consecutive patches along W, then
+// H, then planes, so global reads and writes of a wavefront are contiguous.
+//
+// Knobs (-D constants): NT threads per workgroup, TH x TW outputs per lane,
+// NT_STORE (1: non-temporal stores for the output).
+// Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
+// STR, PAD, DIL, FACT, CP x CQ output.
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define PLANES (CB * CC * FACT)
+#define TILES_H ((CP + TH - 1) / TH)
+#define TILES_W ((CQ + TW - 1) / TW)
+#define ITEMS (PLANES * TILES_H * TILES_W)
+#define IH_T ((TH - 1) * STR + (CR - 1) * DIL + 1)
+#define IW_T ((TW - 1) * STR + (CS - 1) * DIL + 1)
+
+/* 128-bit path: same-size stride-1 convolution whose rows keep 16-byte
+ * alignment; the four centre columns of a patch come in as one vector. */
+#if (TW == 4) && (STR == 1) && (CW % 4 == 0) && (CQ == CW) && (PAD + 4 <= IW_T)
+#define VEC_IN 1
+#else
+#define VEC_IN 0
+#endif
+#if (TW == 4) && (CQ % 4 == 0)
+#define VEC_OUT 1
+#else
+#define VEC_OUT 0
+#endif
+
+extern "C" __global__ __launch_bounds__(NT)
+void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
+                   float* __restrict__ O)
+{
+    const int gid = blockIdx.x * NT + threadIdx.x;
+    if (gid >= ITEMS) return;
+    const int tw = gid % TILES_W;
+    const int th = (gid / TILES_W) % TILES_H;
+    const int plane = gid / (TILES_W * TILES_H);
+    const int b = plane / (CC * FACT);
+    const int co = plane % (CC * FACT);
+    const int ci = co / FACT;
+    const float* x = X + (size_t)(b * CC + ci) * (CH * CW);
+    const float* wp = Wt + (size_t)co * (CR * CS);
+    float* o = O + (size_t)plane * (CP * CQ);
+
+    float wreg[CR][CS];
+#pragma unroll
+    for (int r = 0; r < CR; ++r)
+#pragma unroll
+        for (int s = 0; s < CS; ++s)
+            wreg[r][s] = wp[r * CS + s];
+
+    const int oh0 = th * TH;
+    const int ow0 = tw * TW;
+    const int ih0 = oh0 * STR - PAD;
+    const int iw0 = ow0 * STR - PAD;
+
+    float acc[TH][TW];
+#pragma unroll
+    for (int i = 0; i < TH; ++i)
+#pragma unroll
+        for (int j = 0; j < TW; ++j)
+            acc[i][j] = 0.0f;
+
+#pragma unroll
+    for (int y = 0; y < IH_T; ++y) {
+        const int ih = ih0 + y;
+        const bool row_ok = (unsigned)ih < (unsigned)CH;
+        const float* xr = x + ih * CW;
+        float in[IW_T];
+#if VEC_IN
+        {
+            f32x4 v = (f32x4)(0.0f);
+            if (row_ok) v = *reinterpret_cast<const f32x4*>(xr + ow0);
+#pragma unroll
+            for (int j = 0; j < IW_T; ++j) {
+                if (j >= PAD && j < PAD + 4) {
+                    in[j] = v[(j - PAD) & 3];
+                } else {
+                    const int iw = iw0 + j;
+                    in[j] = (row_ok && (unsigned)iw < (unsigned)CW) ? xr[iw] : 0.0f;
+                }
+            }
+        }
+#else
+#pragma unroll
+        for (int j = 0; j < IW_T; ++j) {
+            const int iw = iw0 + j;
+            in[j] = (row_ok && (unsigned)iw < (unsigned)CW) ? xr[iw] : 0.0f;
+        }
+#endif
+        /* input row y feeds output row i through tap r when y == i*STR + r*DIL */
+#pragma unroll
+        for (int i = 0; i < TH; ++i) {
+#pragma unroll
+            for (int r = 0; r < CR; ++r) {
+                if (y == i * STR + r * DIL) {
+#pragma unroll
+                    for (int j = 0; j < TW; ++j)
+#pragma unroll
+                        for (int s = 0; s < CS; ++s)
+                            acc[i][j] += in[j * STR + s * DIL] * wreg[r][s];
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < TH; ++i) {
+        const int oh = oh0 + i;
+        if (CP % TH != 0 && oh >= CP) continue;
+        float* orow = o + oh * CQ + ow0;
+#if VEC_OUT
+        f32x4 v;
+        v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
+#if NT_STORE
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(orow));
+#else
+        *reinterpret_cast<f32x4*>(orow) = v;
+#endif
+#else
+#pragma unroll
+        for (int j = 0; j < TW; ++j)
+            if (CQ % TW == 0 || ow0 + j < CQ) orow[j] = acc[i][j];
+#endif
+    }
+}

@@ -1,0 +1,39 @@
+// Small helper kernels for gfx950, hiprtc-compiled.
+//
+//   fill_zero_f32   zero-fill of a float buffer; precedes a split-K GEMM whose
+//                   partial sums meet in C with atomics (a kernel rather than
+//                   a memset call so that the launch sequence stays capturable)
+//   zero_pad2d_f32  P[b][c][h][w] = X[b][c][h-PAD][w-PAD] inside, 0 outside
+//                   (flextensor/nn/ops.py:83-117), used when the graph config
+//                   does not inline the padding into the convolution
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+extern "C" __global__ __launch_bounds__(256)
+void fill_zero_f32(float* __restrict__ p, int n)
+{
+    const int n4 = n >> 2;
+    const int stride = gridDim.x * 256;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n4; i += stride)
+        reinterpret_cast<f32x4*>(p)[i] = (f32x4)(0.0f);
+    const int t = (n4 << 2) + blockIdx.x * 256 + threadIdx.x;
+    if (t < n) p[t] = 0.0f;
+}
+
+#ifdef PADK
+/* shape constants: PB planes (batch*channels), CH x CW input, PAD */
+#define PH (CH + 2 * PAD)
+#define PW (CW + 2 * PAD)
+extern "C" __global__ __launch_bounds__(256)
+void zero_pad2d_f32(const float* __restrict__ X, float* __restrict__ P)
+{
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    if (gid >= PB * PH * PW) return;
+    const int w = gid % PW;
+    const int h = (gid / PW) % PH;
+    const int pl = gid / (PW * PH);
+    const int ih = h - PAD, iw = w - PAD;
+    const bool ok = (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+    P[gid] = ok ? X[(size_t)pl * (CH * CW) + ih * CW + iw] : 0.0f;
+}
+#endif

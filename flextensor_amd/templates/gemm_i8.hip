@@ -1,0 +1,216 @@
+// int8 x int8 -> int32 GEMM kernel template for gfx950 (CDNA4), hiprtc-compiled.
+//
+//   C[M][N] = sum_k int32(A[m][k]) * int32(B[n][k])
+//
+// A is [M][K] and B is [N][K], both K-contiguous ("B in K-major layout"), C is
+// row-major int32 — the compute of
+// flextensor/test/test_tvm/legacy/gemm_int8.py:15-21.
+//
+// Knobs (-D constants set by the scheduler from a Config):
+//   MFMA        32 -> v_mfma_i32_32x32x32_i8, 16 -> v_mfma_i32_16x16x64_i8
+//   WAVES_M/N   wavefronts per workgroup along M / N
+//   REP_M/N     MFMA tiles per wavefront along M / N
+//   BK          bytes of K per LDS tile (multiple of the MFMA K)
+//   STAGES      1 or 2 LDS buffers
+//   GROUP_M     tile-traversal group height (L2 locality)
+//   XCD_REMAP   1: consecutive logical tiles stay on one XCD
+//   PAD         LDS row padding in bytes (multiple of 16)
+//   NT_STORE    1: non-temporal stores for C
+//
+// Both operands live in LDS as [rows][BK+PAD] bytes and are read as one
+// 128-bit load per lane per MFMA: lane (i, g) takes the 16 bytes at
+// k = kstep + 16*g of row i, identically for A and B, so whatever order the
+// matrix core assigns to those 16 values inside its K dimension, A and B
+// agree and the integer sum is exact.
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+#if MFMA == 32
+typedef i32x16 acc_t;
+#define NACC 16
+#define MFMA_K 32
+#define MFMA_OP(a, b, c) __builtin_amdgcn_mfma_i32_32x32x32_i8((a), (b), (c), 0, 0, 0)
+#elif MFMA == 16
+typedef i32x4 acc_t;
+#define NACC 4
+#define MFMA_K 64
+#define MFMA_OP(a, b, c) __builtin_amdgcn_mfma_i32_16x16x64_i8((a), (b), (c), 0, 0, 0)
+#else
+#error "MFMA must be 16 or 32"
+#endif
+
+#define BM (WAVES_M * REP_M * MFMA)
+#define BN (WAVES_N * REP_N * MFMA)
+#define NT (WAVES_M * WAVES_N * 64)
+#define SROW (BK + PAD)           /* LDS row stride in bytes */
+#define TILES_M ((M + BM - 1) / BM)
+#define TILES_N ((N + BN - 1) / BN)
+#define KT (K / BK)               /* K % BK == 0 is checked on the host */
+
+#if BK % MFMA_K != 0
+#error "BK must be a multiple of the MFMA K extent"
+#endif
+#if PAD % 16 != 0
+#error "PAD must be a multiple of 16 bytes"
+#endif
+
+#define CHUNKS_ROW (BK / 16)
+#define A_CHUNKS (BM * CHUNKS_ROW)
+#define B_CHUNKS (BN * CHUNKS_ROW)
+#define EA ((A_CHUNKS + NT - 1) / NT)
+#define EB ((B_CHUNKS + NT - 1) / NT)
+
+extern "C" __global__ __launch_bounds__(NT)
+void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ B,
+             int* __restrict__ C)
+{
+    __shared__ __attribute__((aligned(16))) signed char As[STAGES][BM * SROW];
+    __shared__ __attribute__((aligned(16))) signed char Bs[STAGES][BN * SROW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N;
+    const int wn = wave % WAVES_N;
+    const int li = lane % MFMA;
+    const int lg = lane / MFMA;
+
+    const int nblk = TILES_M * TILES_N;
+    int bid = blockIdx.x;
+#if XCD_REMAP
+    if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
+#endif
+    const int grp = bid / (GROUP_M * TILES_N);
+    const int first_m = grp * GROUP_M;
+    const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
+    const int rr = bid % (GROUP_M * TILES_N);
+    const int tile_m = first_m + rr % gsz;
+    const int tile_n = rr / gsz;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+
+    int a_row[EA], a_col[EA], b_row[EB], b_col[EB];
+#pragma unroll
+    for (int e = 0; e < EA; ++e) {
+        const int q = tid + e * NT;
+        a_row[e] = q / CHUNKS_ROW;
+        a_col[e] = (q % CHUNKS_ROW) * 16;
+    }
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+        const int q = tid + e * NT;
+        b_row[e] = q / CHUNKS_ROW;
+        b_col[e] = (q % CHUNKS_ROW) * 16;
+    }
+
+    i32x4 areg[EA], breg[EB];
+
+    auto load_global = [&](int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int e = 0; e < EA; ++e) {
+            const int m = m0 + a_row[e];
+            bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
+            if (M % BM != 0) ok = ok && (m < M);
+            if (ok) areg[e] = *reinterpret_cast<const i32x4*>(A + (size_t)m * K + k0 + a_col[e]);
+            else areg[e] = (i32x4)(0);
+        }
+#pragma unroll
+        for (int e = 0; e < EB; ++e) {
+            const int n = n0 + b_row[e];
+            bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
+            if (N % BN != 0) ok = ok && (n < N);
+            if (ok) breg[e] = *reinterpret_cast<const i32x4*>(B + (size_t)n * K + k0 + b_col[e]);
+            else breg[e] = (i32x4)(0);
+        }
+    };
+
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int e = 0; e < EA; ++e)
+            if ((A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS))
+                *reinterpret_cast<i32x4*>(&As[buf][a_row[e] * SROW + a_col[e]]) = areg[e];
+#pragma unroll
+        for (int e = 0; e < EB; ++e)
+            if ((B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS))
+                *reinterpret_cast<i32x4*>(&Bs[buf][b_row[e] * SROW + b_col[e]]) = breg[e];
+    };
+
+    acc_t acc[REP_M][REP_N];
+#pragma unroll
+    for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j)
+            acc[i][j] = (acc_t)(0);
+
+    auto compute = [&](int buf) {
+        const signed char* as = &As[buf][(wm * REP_M * MFMA + li) * SROW + 16 * lg];
+        const signed char* bs = &Bs[buf][(wn * REP_N * MFMA + li) * SROW + 16 * lg];
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += MFMA_K) {
+            i32x4 a[REP_M], b[REP_N];
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+                a[i] = *reinterpret_cast<const i32x4*>(as + i * MFMA * SROW + kk);
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+                b[j] = *reinterpret_cast<const i32x4*>(bs + j * MFMA * SROW + kk);
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+                for (int j = 0; j < REP_N; ++j)
+                    acc[i][j] = MFMA_OP(a[i], b[j], acc[i][j]);
+        }
+    };
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+#if STAGES == 2
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) load_global(kt + 1);
+        compute(cur);
+        if (kt + 1 < KT) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+#else
+    for (int kt = 0; kt < KT; ++kt) {
+        if (kt + 1 < KT) load_global(kt + 1);
+        compute(0);
+        __syncthreads();
+        if (kt + 1 < KT) {
+            store_lds(0);
+            __syncthreads();
+        }
+    }
+#endif
+
+#pragma unroll
+    for (int i = 0; i < REP_M; ++i) {
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j) {
+            const int n = n0 + (wn * REP_N + j) * MFMA + li;
+#pragma unroll
+            for (int v = 0; v < NACC; ++v) {
+#if MFMA == 32
+                const int row = 8 * (v / 4) + 4 * lg + (v % 4);
+#else
+                const int row = 4 * lg + v;
+#endif
+                const int m = m0 + (wm * REP_M + i) * MFMA + row;
+                bool ok = true;
+                if (M % BM != 0) ok = ok && (m < M);
+                if (N % BN != 0) ok = ok && (n < N);
+                if (ok) {
+#if NT_STORE
+                    __builtin_nontemporal_store(acc[i][j][v], C + (size_t)m * N + n);
+#else
+                    C[(size_t)m * N + n] = acc[i][j][v];
+#endif
+                }
+            }
+        }
+    }
+}

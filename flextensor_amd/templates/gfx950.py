@@ -1,0 +1,437 @@
+"""gfx950 (MI355X) kernel templates: schedule space and config -> kernel.
+
+Where the reference turns a config dict into TVM schedule primitives
+(flextensor/templates/cuda.py:390-661 for GPUs, templates/cpu.py:316-518 for
+CPUs), this module turns the same dict into the ``-D`` constants of a
+hand-written HIP kernel template plus launch geometry. Nothing here touches a
+device: lowering is pure Python and can be unit-tested on a CPU.
+
+Operator kinds and the template each one lowers to:
+
+  gemm                   igemm_f32.hip  MODE 0 (MODE 2 for transposeB)
+  conv2d_nchw            igemm_f32.hip  MODE 1 (implicit GEMM, padding folded
+                                         into the gather; or PAD=0 over a
+                                         materialised padded tensor)
+  gemm_int8              gemm_i8.hip
+  depthwise_conv2d_nchw  depthwise_f32.hip (direct)
+  zero_pad2d             elementwise.hip   (only when not inlined)
+
+Meaning of the config keys: see flextensor_amd/space.py.
+"""
+import os
+
+from ..space import (Space, SplitSpace, TileSplitSpace, LaneTileSpace, UnrollSpace, EnumSpace)
+from ..utils import ceil_div
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+LDS_BYTES = 160 * 1024        # per workgroup on gfx950
+MAX_ACC_REGS = 256            # accumulation VGPRs per lane
+MAX_THREADS = 1024
+NUM_XCD = 8
+
+
+class InvalidConfig(ValueError):
+    """The config does not describe a kernel this template can build."""
+
+
+_SOURCES = {}
+
+
+def template_source(name):
+    if name not in _SOURCES:
+        with open(os.path.join(_HERE, name), "r") as f:
+            _SOURCES[name] = f.read()
+    return _SOURCES[name]
+
+
+class KernelSpec(object):
+    """One kernel of a plan, fully determined on the host.
+
+    template     file name of the HIP source
+    kernel       extern "C" symbol
+    defines      dict of -D constants
+    grid, block  launch geometry
+    args         list of argument descriptors: ("buf", name) for a device
+                 buffer bound by the plan, ("i32", value) / ("i64", value) /
+                 ("u32", value) for scalars
+    """
+
+    def __init__(self, template, kernel, defines, grid, block, args, lds_bytes=0, note=""):
+        self.template = template
+        self.kernel = kernel
+        self.defines = dict(defines)
+        self.grid = tuple(grid)
+        self.block = tuple(block)
+        self.args = list(args)
+        self.lds_bytes = lds_bytes
+        self.note = note
+
+    def options(self):
+        return ["-D%s=%s" % (k, v) for k, v in sorted(self.defines.items())]
+
+    def source(self):
+        return template_source(self.template)
+
+    def __repr__(self):
+        return "KernelSpec(%s %s grid=%s block=%s)" % (self.kernel, self.defines, self.grid, self.block)
+
+
+# --------------------------------------------------------------------------
+# GEMM view of an operator
+# --------------------------------------------------------------------------
+
+class GemmView(object):
+    """M, N, K and addressing mode of a contraction-shaped operator."""
+
+    def __init__(self, op):
+        kind = op.kind
+        self.kind = kind
+        self.conv = None
+        if kind == "gemm":
+            if op.attrs.get("transposeA"):
+                raise NotImplementedError("transposeA is not on the tuned path")
+            self.M, self.N = op.axis[0].extent, op.axis[1].extent
+            self.K = op.reduce_axis[0].extent
+            self.mode = 2 if op.attrs.get("transposeB") else 0
+            self.dtype = "float32"
+        elif kind == "gemm_int8":
+            self.M, self.N = op.axis[0].extent, op.axis[1].extent
+            self.K = op.reduce_axis[0].extent
+            self.mode = 0
+            self.dtype = "int8"
+        elif kind == "conv2d_nchw":
+            a = op.attrs
+            if a["groups"] != 1:
+                raise NotImplementedError("grouped conv2d is not on the tuned path")
+            if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
+                    or a["dilation"][0] != a["dilation"][1]:
+                raise NotImplementedError("anisotropic stride/padding/dilation")
+            b, kout, p, q = [x.extent for x in op.axis]
+            c = op.reduce_axis[0].extent
+            s = op.reduce_axis[1].extent  # rw
+            r = op.reduce_axis[2].extent  # rh
+            _, _, h, w = a["in_shape"]
+            self.M, self.N, self.K = kout, b * p * q, c * r * s
+            self.mode = 1
+            self.dtype = "float32"
+            self.conv = dict(CB=b, CC=c, CH=h, CW=w, CR=r, CS=s, CSTR=a["stride"][0],
+                             CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
+        else:
+            raise InvalidConfig("operator kind %s has no GEMM view" % kind)
+        # K as the kernels iterate it: fp32 pads the tail up to a multiple of
+        # 16 with predicated (zero) loads; int8 needs whole 16-byte K chunks.
+        self.KP = self.K if self.dtype == "int8" else ceil_div(self.K, 16) * 16
+
+
+F32_BK = (8, 16, 32, 64)
+I8_BK = (64, 128, 256)
+
+
+def _gemm_space(view):
+    space = Space()
+    i8 = view.dtype == "int8"
+    reps = (1, 2, 3, 4, 6, 8)
+    space.add_subspace("split_m_0", TileSplitSpace(view.M, reps=reps), "spatial")
+    space.add_subspace("split_n_1", TileSplitSpace(view.N, reps=reps), "spatial")
+    bks = I8_BK if i8 else F32_BK
+    max_split = 1 if i8 else 16
+
+    def keep(e):
+        return e[2] in bks and e[0] <= max_split
+
+    rs = SplitSpace(3, view.KP, keep=keep)
+    if rs.size == 0:
+        raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
+    space.add_subspace("split_k_0", rs, "reduce")
+    space.add_subspace("unroll", UnrollSpace([1, 2], explicit=True), "unroll")
+    space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
+    space.add_subspace("xcd_remap", EnumSpace([[0], [1]]), "reorder")
+    return space
+
+
+def _depthwise_space(op):
+    space = Space()
+    b, c, p, q = [x.extent for x in op.axis]
+    space.add_subspace("split_b_0", LaneTileSpace(b, [1]), "spatial")
+    space.add_subspace("split_c_1", LaneTileSpace(c, [1]), "spatial")
+    space.add_subspace("split_h_2", LaneTileSpace(p, [1, 2, 4, 7, 8, 14]), "spatial")
+    space.add_subspace("split_w_3", LaneTileSpace(q, [1, 2, 4]), "spatial")
+    space.add_subspace("waves", EnumSpace([[1], [2], [4], [8]]), "fuse")
+    return space
+
+
+def generate_space(op):
+    """Schedule space of one operator for gfx950."""
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+        return _gemm_space(GemmView(op))
+    if op.kind == "depthwise_conv2d_nchw":
+        return _depthwise_space(op)
+    if op.kind == "zero_pad2d":
+        return Space()
+    raise InvalidConfig("no gfx950 template for operator kind %s" % op.kind)
+
+
+# --------------------------------------------------------------------------
+# special (task-level enumerated) knobs
+# --------------------------------------------------------------------------
+
+SPECIAL_DEFAULTS = {
+    "lds_pad": [4, 8],     # fp32: [APAD, BPAD] floats; int8: [PAD bytes / 4, -]
+    "nt_store": [0],
+}
+
+
+def special_knobs(kind):
+    """Enumerated knobs a task of this operator kind carries by default; they
+    are attached with Task.set_specific_space and searched at graph level."""
+    if kind in ("gemm", "conv2d_nchw"):
+        return {"lds_pad": [[4, 8], [4, 4], [0, 0], [4, 16], [8, 8]]}
+    if kind == "gemm_int8":
+        return {"lds_pad": [[4, 0], [8, 0], [0, 0]], "nt_store": [[0], [1]]}
+    if kind == "depthwise_conv2d_nchw":
+        return {"nt_store": [[0], [1]]}
+    return {}
+
+
+def _special(graph_special, name):
+    if graph_special and name in graph_special:
+        return list(graph_special[name])
+    return list(SPECIAL_DEFAULTS[name])
+
+
+# --------------------------------------------------------------------------
+# lowering
+# --------------------------------------------------------------------------
+
+def _one(config, key, n, what):
+    lst = config.get(key) or []
+    if len(lst) != n:
+        raise InvalidConfig("%s: expected %d '%s' entries, got %d" % (what, n, key, len(lst)))
+    return lst
+
+
+def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False):
+    view = GemmView(op)
+    sp = _one(config, "spatial", 2, op.kind)
+    rd = _one(config, "reduce", 1, op.kind)
+    (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
+    splitk, kiters, bk = [int(x) for x in rd[0]]
+    stages = int((config.get("unroll") or [[2, 1]])[0][0])
+    group_m = int((config.get("fuse") or [[4]])[0][0])
+    xcd = int((config.get("reorder") or [[1]])[0][0])
+    i8 = view.dtype == "int8"
+
+    if mfm != mfn or mfm not in (16, 32):
+        raise InvalidConfig("MFMA edge must be 16 or 32 and equal on both axes")
+    if min(wm, rm, wn, rn, splitk, kiters, bk, group_m) < 1:
+        raise InvalidConfig("non-positive factor")
+    if stages not in (1, 2):
+        raise InvalidConfig("LDS stages must be 1 or 2")
+    nwaves = wm * wn
+    if nwaves * 64 > MAX_THREADS:
+        raise InvalidConfig("more than 16 wavefronts per workgroup")
+    bm, bn = wm * rm * mfm, wn * rn * mfn
+    if gm != ceil_div(view.M, bm) or gn != ceil_div(view.N, bn):
+        raise InvalidConfig("grid level does not match ceil(extent / tile)")
+    nacc = rm * rn * (mfm * mfm // 64)
+    if nacc > MAX_ACC_REGS:
+        raise InvalidConfig("accumulators need %d registers per lane" % nacc)
+    if splitk * kiters * bk != view.KP:
+        raise InvalidConfig("reduce split does not multiply to K")
+    nt = nwaves * 64
+    D = dict(M=view.M, N=view.N, K=view.K, KP=view.KP, MFMA=mfm, WAVES_M=wm, WAVES_N=wn, REP_M=rm,
+             REP_N=rn, BK=bk, STAGES=stages, GROUP_M=group_m, XCD_REMAP=xcd)
+
+    if i8:
+        if splitk != 1:
+            raise InvalidConfig("int8 GEMM does not split K across workgroups")
+        mfma_k = 32 if mfm == 32 else 64
+        if bk % mfma_k != 0 or view.K % 16 != 0:
+            raise InvalidConfig("BK must be a multiple of the MFMA K extent")
+        pad = int(_special(special, "lds_pad")[0]) * 4
+        if pad % 16 != 0:
+            raise InvalidConfig("int8 LDS padding must be a multiple of 16 bytes")
+        lds = stages * (bm + bn) * (bk + pad)
+        if lds > LDS_BYTES:
+            raise InvalidConfig("LDS tile needs %d bytes" % lds)
+        D.update(PAD=pad, NT_STORE=int(_special(special, "nt_store")[0]))
+        grid = (gm * gn, 1, 1)
+        spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
+                          [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])
+        return [spec]
+
+    kblk = 4 * (64 // mfm)
+    if bk % kblk != 0:
+        raise InvalidConfig("BK must be a multiple of %d for this MFMA shape" % kblk)
+    apad, bpad = [int(x) for x in _special(special, "lds_pad")[:2]]
+    if apad % 4 != 0 or bpad % 4 != 0:
+        raise InvalidConfig("fp32 LDS padding must keep 16-byte alignment")
+    av = 4 if view.K % 4 == 0 else 1
+    if view.mode == 0:
+        bv = 4 if view.N % 4 == 0 else 1
+    elif view.mode == 2:
+        bv = av
+    else:
+        bv = 1
+    sa = bk + apad
+    if view.mode == 2:
+        lds_b = bn * sa
+    else:
+        lds_b = bk * (bn + bpad)
+    lds = stages * 4 * (bm * sa + lds_b)
+    if lds > LDS_BYTES:
+        raise InvalidConfig("LDS tile needs %d bytes" % lds)
+    # staging registers for the global->LDS copy must stay reasonable
+    ea = ceil_div(bm * bk // av, nt)
+    eb = ceil_div((bn * bk) // bv, nt)
+    if (ea * av + eb * bv) > 128:
+        raise InvalidConfig("global->LDS staging needs too many registers")
+    D.update(MODE=view.mode, SPLITK=splitk, APAD=apad, BPAD=bpad, AV=av, BV=bv)
+    specs = []
+    if view.mode == 1:
+        conv = dict(view.conv)
+        if materialized_pad:
+            conv["CH"] += 2 * conv["CPAD"]
+            conv["CW"] += 2 * conv["CPAD"]
+            conv["CPAD"] = 0
+        D.update(conv)
+        # A = weight, B = image
+        a_name, b_name = in_names[1], in_names[0]
+    else:
+        a_name, b_name = in_names[0], in_names[1]
+    if splitk > 1:
+        nout = view.M * view.N
+        specs.append(KernelSpec("elementwise.hip", "fill_zero_f32", {},
+                                (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
+                                [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
+    grid = (gm * gn * splitk, 1, 1)
+    specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt, 1, 1),
+                            [("buf", a_name), ("buf", b_name), ("buf", out_name)]))
+    return specs
+
+
+def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=False):
+    sp = _one(config, "spatial", 4, op.kind)
+    th, tw = int(sp[2][3]), int(sp[3][3])
+    if int(sp[0][3]) != 1 or int(sp[1][3]) != 1:
+        raise InvalidConfig("depthwise lanes own one batch entry and one channel")
+    waves = int((config.get("fuse") or [[4]])[0][0])
+    if waves < 1 or waves * 64 > MAX_THREADS:
+        raise InvalidConfig("bad wavefront count")
+    a = op.attrs
+    if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
+            or a["dilation"][0] != a["dilation"][1]:
+        raise NotImplementedError("anisotropic stride/padding/dilation")
+    b, cout, p, q = [x.extent for x in op.axis]
+    s_ext = op.reduce_axis[0].extent  # rw
+    r_ext = op.reduce_axis[1].extent  # rh
+    _, c, h, w = a["in_shape"]
+    if th < 1 or tw < 1 or th > p or tw > q:
+        raise InvalidConfig("lane patch larger than the output plane")
+    if int(sp[2][0]) != ceil_div(p, th) or int(sp[3][0]) != ceil_div(q, tw):
+        raise InvalidConfig("grid level does not match ceil(extent / patch)")
+    pad = a["padding"][0]
+    if materialized_pad:
+        h, w, pad = h + 2 * pad, w + 2 * pad, 0
+    ih_t = (th - 1) * a["stride"][0] + (r_ext - 1) * a["dilation"][0] + 1
+    iw_t = (tw - 1) * a["stride"][0] + (s_ext - 1) * a["dilation"][0] + 1
+    if th * tw + iw_t + r_ext * s_ext > 200:
+        raise InvalidConfig("lane patch needs too many registers")
+    nt = waves * 64
+    items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
+    D = dict(NT=nt, TH=th, TW=tw, NT_STORE=int(_special(special, "nt_store")[0]),
+             CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=a["stride"][0], PAD=pad,
+             DIL=a["dilation"][0], FACT=a["factor"], CP=p, CQ=q)
+    del ih_t
+    return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(items, nt), 1, 1),
+                       (nt, 1, 1),
+                       [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
+
+
+def _lower_pad(op, out_name, in_names):
+    b, c, ph, pw = [x.extent for x in op.axis]
+    pt, pb, pl, pr = op.attrs["padding"]
+    if not (pt == pb == pl == pr):
+        raise NotImplementedError("asymmetric padding")
+    h, w = ph - 2 * pt, pw - 2 * pt
+    D = dict(PADK=1, PB=b * c, CH=h, CW=w, PAD=pt)
+    n = b * c * ph * pw
+    return [KernelSpec("elementwise.hip", "zero_pad2d_f32", D, (ceil_div(n, 256), 1, 1),
+                       (256, 1, 1), [("buf", in_names[0]), ("buf", out_name)])]
+
+
+def lower(op, config, special, out_name, in_names, materialized_pad=False):
+    """Config of one operator -> list of KernelSpec (raises InvalidConfig)."""
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+        return _lower_gemm(op, config, special, out_name, in_names, materialized_pad)
+    if op.kind == "depthwise_conv2d_nchw":
+        return _lower_depthwise(op, config, special, out_name, in_names, materialized_pad)
+    if op.kind == "zero_pad2d":
+        return _lower_pad(op, out_name, in_names)
+    raise InvalidConfig("no gfx950 template for operator kind %s" % op.kind)
+
+
+# --------------------------------------------------------------------------
+# default (untuned) configs
+# --------------------------------------------------------------------------
+
+def _empty_config():
+    return {k: [] for k in Space.valid_type_keys}
+
+
+def default_config(op):
+    """A reasonable untuned config: what schedule_with_config falls back to
+    when a task has no tuned entry, and the seed point of the search."""
+    cfg = _empty_config()
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+        view = GemmView(op)
+        i8 = view.dtype == "int8"
+
+        def tile(extent, want):
+            mf = 32 if extent >= 32 else 16
+            t = mf
+            w, r = 1, 1
+            while w * r * mf * 2 <= want and w * r * mf * 2 <= max(extent, mf):
+                if w < 2:
+                    w *= 2
+                else:
+                    r *= 2
+            del t
+            return [ceil_div(extent, w * r * mf), w, r, mf]
+
+        want = 256 if i8 else 128
+        tm, tn = tile(view.M, want), tile(view.N, want)
+        mf = min(tm[3], tn[3])
+        for t, ext in ((tm, view.M), (tn, view.N)):
+            if t[3] != mf:
+                t[2] *= t[3] // mf
+                t[3] = mf
+            t[0] = ceil_div(ext, t[1] * t[2] * t[3])
+        cfg["spatial"] = [tm, tn]
+        bks = I8_BK if i8 else F32_BK
+        kblk = (32 if mf == 32 else 64) if i8 else 4 * (64 // mf)
+        bk = None
+        for cand in sorted(bks, reverse=True):
+            if view.KP % cand == 0 and cand % kblk == 0 and cand <= (64 if i8 else 16):
+                bk = cand
+                break
+        if bk is None:
+            for cand in sorted(bks):
+                if view.KP % cand == 0 and cand % kblk == 0:
+                    bk = cand
+                    break
+        if bk is None:
+            raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
+        cfg["reduce"] = [[1, view.KP // bk, bk]]
+        cfg["unroll"] = [[2, 1]]
+        cfg["fuse"] = [[4]]
+        cfg["reorder"] = [[1]]
+    elif op.kind == "depthwise_conv2d_nchw":
+        b, c, p, q = [x.extent for x in op.axis]
+        th = 4 if p >= 4 else 1
+        tw = 4 if q >= 4 else 1
+        cfg["spatial"] = [[b, 1, 1, 1], [c, 1, 1, 1], [ceil_div(p, th), 1, 1, th],
+                          [ceil_div(q, tw), 1, 1, tw]]
+        cfg["fuse"] = [[4]]
+    return cfg

@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the tuned hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+
+One step = one run of the tuned kernel plan of the headline workload
+(conv2d NCHW fp32, N=1, C=64, H=W=56, K=64, 3x3, stride 1, pad 1) over
+seeded synthetic inputs that are resident in HBM before the timed region.
+W untimed steps, then exactly K steps between two device synchronisations.
+Prints ONE JSON line with the whole-job throughput (`value`, TFLOP/s), the
+roofline position of the dominant kernel measured with HIP events on the
+launch stream, the same figures for the other benchmark configurations
+(`per_config`) and the CPU baseline (the multi-threaded CPU port of the
+reference's llvm path, oracle/cpu_baseline.c) timed on this host.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks (dense)
+PEAK_F32_TFLOPS = 157.3
+PEAK_I8_TOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = [
+    # name, task key, op count (FLOP or OP), compulsory bytes, bound, dtype
+    ("gemm_f32_1024", "gemm_gemm_(1024, 1024, 1024)_rocm(0)", 2 * 1024 ** 3, 12582912, "mfma", "f32"),
+    ("conv2d_1x64x56x56_k64_3x3", "conv2d_baseline0_(1, 64, 56, 56, 64, 3, 1, 1, 1, 1)_rocm(0)",
+     231211008, 1753088, "mfma", "f32"),
+    ("conv2d_8x256x14x14_k512_3x3", "conv2d_baseline1_(8, 256, 14, 14, 512, 3, 1, 1, 1, 1)_rocm(0)",
+     3699376128, 9535488, "mfma", "f32"),
+    ("conv2d_8x512x7x7_k2048_1x1", "conv2d_baseline2_(8, 512, 7, 7, 2048, 1, 1, 0, 1, 1)_rocm(0)",
+     822083584, 8208384, "mfma", "f32"),
+    ("depthwise_8x512x28x28_3x3", "conv2d_depthwise_(8, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)",
+     57802752, 25708544, "hbm", "f32"),
+    ("gemm_i8_4096", "gemm_gemm_int8_(4096, 4096, 4096)_rocm(0)", 2 * 4096 ** 3, 100663296, "mfma", "i8"),
+]
+HEADLINE = 1  # configs[1] of BASELINE.json
+
+
+def roofline(bound, dtype, ops, nbytes, ms):
+    if bound == "hbm":
+        achieved = nbytes / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": achieved / PEAK_HBM_GBS, "traffic": None}
+    peak = PEAK_I8_TOPS if dtype == "i8" else PEAK_F32_TFLOPS
+    achieved = ops / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": achieved, "peak": peak,
+            "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak, "traffic": None}
+
+
+def gpu_workload(key, seed=0):
+    """(built plan, buffer sets, plan) for a task, using its shipped tuned config."""
+    from flextensor_amd.measure import get_measurer
+    from flextensor_amd.scheduler import schedule_with_config
+    from flextensor_amd.tuned import lookup
+    from flextensor_amd.utils import Config
+    cfg = lookup(key) or Config([], None)
+    s, _ = schedule_with_config(key, cfg)
+    m = get_measurer(key, seed)
+    built = s.build()
+    return built, m, s
+
+
+def kernel_ms(built, m, iters=200, warmup=20):
+    """Mean duration of one plan run, HIP events on the launch stream."""
+    import torch
+    first = m.sets[0]
+    built(*first)
+    torch.cuda.synchronize()
+    ok, metric = m.check(first[-1])
+    if not ok:
+        raise RuntimeError("tuned plan fails the correctness gate (metric %g)" % metric)
+    return built.time(m.sets, warmup=warmup, iters=iters), metric
+
+
+def cpu_baseline_for(name, key, ops, budget_s):
+    """Time the multi-threaded CPU port on the same seeded workload.
+    Returns (ms per pass, threads, sample description)."""
+    import numpy as np
+    from flextensor_amd.measure import seeded_inputs
+    from flextensor_amd.task import TASK_TABLE
+    from oracle import oracle as o  # CPU baseline leg: the only use of the oracle here
+    task = TASK_TABLE[key]
+    _, bufs = task.func(*task.args)
+    host = seeded_inputs(bufs, 0)
+    threads = o.baseline_threads()
+    frac = 1.0
+    if name.startswith("gemm_f32"):
+        out = np.empty(bufs[-1].shape, np.float32)
+        fn = lambda: o.baseline_gemm_f32(host[0], host[1], out, 256)  # noqa: E731
+    elif name.startswith("gemm_i8"):
+        out = np.zeros(bufs[-1].shape, np.int32)
+        rows = 256
+        frac = rows / bufs[-1].shape[0]
+        fn = lambda: o.baseline_gemm_i8(host[0], host[1], out, 0, rows)  # noqa: E731
+    elif name.startswith("conv2d"):
+        a = task.args
+        out = np.empty(bufs[-1].shape, np.float32)
+        scratch = np.empty((a[0], a[1], a[2] + 2 * a[7], a[3] + 2 * a[7]), np.float32)
+        fn = lambda: o.baseline_conv2d(host[0], host[1], out, scratch, a[6], a[7], a[8])  # noqa: E731
+    else:
+        a = task.args
+        out = np.empty(bufs[-1].shape, np.float32)
+        scratch = np.empty((a[0], a[1], a[2] + 2 * a[7], a[3] + 2 * a[7]), np.float32)
+        fn = lambda: o.baseline_depthwise(host[0], host[1], out, scratch, a[6], a[7], a[8])  # noqa: E731
+    fn()  # warm-up
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        fn()
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or n >= 2000:
+            break
+    ms = el / n * 1e3 / frac
+    sample = "%d passes of the full workload" % n if frac == 1.0 else \
+        "%d passes over the first %d output rows, scaled to the full matrix" % (n, rows)
+    return ms, threads, sample
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the tuned kernels are single-device and nothing "
+              "here shards across GPUs; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from flextensor_amd import runtime as rt
+    from flextensor_amd.plan import current_stream
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    props = rt.device_props(0)
+
+    name, key, ops, nbytes, bound, dtype = WORKLOADS[HEADLINE]
+    built, m, plan = gpu_workload(key)
+    # ---- headline: W untimed steps, exactly K timed steps -----------------
+    launches = built.launches(m.sets[0])
+    stream = current_stream()
+    for _ in range(args.warmup):
+        rt.launch_seq(launches, stream=stream)
+    torch.cuda.synchronize()
+    seq = launches * args.steps          # one C call enqueues all K steps
+    arr = rt._desc_array(seq)
+    t0 = time.perf_counter()
+    rt._check(rt.lib().ftr_launch_seq(arr, len(seq), ctypes.c_void_p(stream)), "ftr_launch_seq")
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = ops / (ms_per_step * 1e-3) / 1e12
+    ok, metric = m.check(m.sets[0][-1])
+    if not ok:
+        raise RuntimeError("headline plan fails the correctness gate (metric %g)" % metric)
+    k_ms, _ = kernel_ms(built, m, iters=max(args.steps // 4, 50))
+    roof = roofline(bound, dtype, ops, nbytes, k_ms)
+    roof["kernel"] = plan.specs[-1].kernel
+    roof["kernel_ms"] = k_ms
+    built.close()
+
+    per_config = []
+    if not args.only_headline:
+        for (wname, wkey, wops, wbytes, wbound, wdtype) in WORKLOADS:
+            b, mm, pl = gpu_workload(wkey)
+            ms, met = kernel_ms(b, mm, iters=100 if wdtype == "i8" else 300)
+            r = roofline(wbound, wdtype, wops, wbytes, ms)
+            entry = {"workload": wname, "ms": ms, "dtype": wdtype,
+                     "throughput": wops / (ms * 1e-3) / 1e12,
+                     "throughput_unit": "TOP/s" if wdtype == "i8" else "TFLOP/s",
+                     "roofline": r, "check": met,
+                     "kernels": [s.kernel for s in pl.specs],
+                     "config": json.loads(json.dumps(pl.configs))}
+            b.close()
+            per_config.append(entry)
+
+    cpu = None
+    if not args.no_cpu:
+        ms, threads, sample = cpu_baseline_for(name, key, ops, args.cpu_seconds)
+        cpu = {"value": ops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "cores": threads,
+               "kind": "port", "ms": ms, "sample": sample + " (oracle/cpu_baseline.c, the "
+               "reference's llvm template structure in C/OpenMP; TVM itself is unavailable)"}
+        if not args.only_headline:
+            for entry, (wname, wkey, wops, _, _, _) in zip(per_config, WORKLOADS):
+                if wname == name:
+                    entry["cpu_ms"], entry["cpu_cores"] = ms, threads
+                    continue
+                cms, cth, _ = cpu_baseline_for(wname, wkey, wops, 1.0)
+                entry["cpu_ms"], entry["cpu_cores"] = cms, cth
+
+    line = {
+        "metric": "best-config TFLOPS + % of MI355X roofline per op vs CPU llvm baseline",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": name + " (BASELINE.json configs[1])", "task_key": key,
+                   "tuned_config": json.loads(json.dumps(plan.configs)),
+                   "device": props["name"], "arch": props["arch"]},
+        "roofline": roof, "cpu_baseline": cpu, "per_config": per_config,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

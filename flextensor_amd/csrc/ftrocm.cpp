@@ -40,9 +40,11 @@ int fail(const char *fmt, ...) {
 #define FTR_HIP(call)                                                         \
     do {                                                                      \
         hipError_t e_ = (call);                                               \
-        if (e_ != hipSuccess)                                                 \
+        if (e_ != hipSuccess) {                                               \
+            (void)hipGetLastError(); /* do not leave a sticky error behind */ \
             return fail("%s failed: %s (%d)", #call, hipGetErrorString(e_),   \
                         (int)e_);                                             \
+        }                                                                     \
     } while (0)
 
 int launch_one(const ftr_launch_desc_t &d, hipStream_t s) {
@@ -133,6 +135,7 @@ int ftr_module_load(const void *code, size_t size, const char *kernel_name,
     hipError_t e = hipModuleGetFunction(&f, m, kernel_name);
     if (e != hipSuccess) {
         (void)hipModuleUnload(m);
+        (void)hipGetLastError();
         return fail("kernel '%s' not found in code object: %s", kernel_name,
                     hipGetErrorString(e));
     }
@@ -246,8 +249,10 @@ int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc) return 1;
-    if (e != hipSuccess)
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
         return fail("timing failed: %s (%d)", hipGetErrorString(e), (int)e);
+    }
     *ms_mean = ms / (float)iters;
     return 0;
 }

@@ -305,7 +305,7 @@ class TileSplitSpace(SubSpace):
                     padded = grid * tile
                     if grid > 1 and (padded - extent) > max_waste * extent:
                         continue
-                    if grid == 1 and tile >= 2 * extent and tile > mf:
+                    if grid == 1 and tile - extent >= mf:
                         continue  # a smaller tile covers the axis as well
                     ents.append([grid, w, r, mf])
         ents.sort(key=lambda e: (e[1] * e[2] * e[3], e[3], e[1]))

@@ -15,6 +15,25 @@
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
 // STR, PAD, DIL, FACT, CP x CQ output.
 
+/* Constants arrive as -DFT_<NAME>=value: single-letter macros on the command line
+ * would be visible to (and break) the runtime-compilation built-in headers. */
+#define NT FT_NT
+#define TH FT_TH
+#define TW FT_TW
+#define NT_STORE FT_NT_STORE
+#define CB FT_CB
+#define CC FT_CC
+#define CH FT_CH
+#define CW FT_CW
+#define CR FT_CR
+#define CS FT_CS
+#define STR FT_STR
+#define PAD FT_PAD
+#define DIL FT_DIL
+#define FACT FT_FACT
+#define CP FT_CP
+#define CQ FT_CQ
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define PLANES (CB * CC * FACT)

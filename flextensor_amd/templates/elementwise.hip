@@ -20,7 +20,11 @@ void fill_zero_f32(float* __restrict__ p, int n)
     if (t < n) p[t] = 0.0f;
 }
 
-#ifdef PADK
+#ifdef FT_PADK
+#define PB FT_PB
+#define CH FT_CH
+#define CW FT_CW
+#define PAD FT_PAD
 /* shape constants: PB planes (batch*channels), CH x CW input, PAD */
 #define PH (CH + 2 * PAD)
 #define PW (CW + 2 * PAD)

@@ -23,6 +23,24 @@
 // matrix core assigns to those 16 values inside its K dimension, A and B
 // agree and the integer sum is exact.
 
+/* Constants arrive as -DFT_<NAME>=value: single-letter macros on the command line
+ * would be visible to (and break) the runtime-compilation built-in headers. */
+#define M FT_M
+#define N FT_N
+#define K FT_K
+#define KP FT_KP
+#define MFMA FT_MFMA
+#define WAVES_M FT_WAVES_M
+#define WAVES_N FT_WAVES_N
+#define REP_M FT_REP_M
+#define REP_N FT_REP_N
+#define BK FT_BK
+#define STAGES FT_STAGES
+#define GROUP_M FT_GROUP_M
+#define XCD_REMAP FT_XCD_REMAP
+#define PAD FT_PAD
+#define NT_STORE FT_NT_STORE
+
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
 
@@ -46,7 +64,9 @@ typedef i32x4 acc_t;
 #define SROW (BK + PAD)           /* LDS row stride in bytes */
 #define TILES_M ((M + BM - 1) / BM)
 #define TILES_N ((N + BN - 1) / BN)
-#define KT (K / BK)               /* K % BK == 0 is checked on the host */
+/* KP = K rounded up to a multiple of 64 (host checks KP % BK == 0 and
+ * K % 16 == 0); chunks beyond K are zero-filled by the load predicate. */
+#define KT (KP / BK)
 
 #if BK % MFMA_K != 0
 #error "BK must be a multiple of the MFMA K extent"
@@ -113,6 +133,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             const int m = m0 + a_row[e];
             bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
             if (M % BM != 0) ok = ok && (m < M);
+            if (KP != K) ok = ok && (k0 + a_col[e] < K);
             if (ok) areg[e] = *reinterpret_cast<const i32x4*>(A + (size_t)m * K + k0 + a_col[e]);
             else areg[e] = (i32x4)(0);
         }
@@ -121,6 +142,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             const int n = n0 + b_row[e];
             bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
             if (N % BN != 0) ok = ok && (n < N);
+            if (KP != K) ok = ok && (k0 + b_col[e] < K);
             if (ok) breg[e] = *reinterpret_cast<const i32x4*>(B + (size_t)n * K + k0 + b_col[e]);
             else breg[e] = (i32x4)(0);
         }

@@ -68,7 +68,7 @@ class KernelSpec(object):
         self.note = note
 
     def options(self):
-        return ["-D%s=%s" % (k, v) for k, v in sorted(self.defines.items())]
+        return ["-DFT_%s=%s" % (k, v) for k, v in sorted(self.defines.items())]
 
     def source(self):
         return template_source(self.template)
@@ -120,8 +120,10 @@ class GemmView(object):
         else:
             raise InvalidConfig("operator kind %s has no GEMM view" % kind)
         # K as the kernels iterate it: fp32 pads the tail up to a multiple of
-        # 16 with predicated (zero) loads; int8 needs whole 16-byte K chunks.
-        self.KP = self.K if self.dtype == "int8" else ceil_div(self.K, 16) * 16
+        # 16 (int8: 64) with predicated zero loads; int8 needs K % 16 == 0.
+        if min(self.M, self.N, self.K) < 1:
+            raise InvalidConfig("empty operator: M, N, K = %d, %d, %d" % (self.M, self.N, self.K))
+        self.KP = ceil_div(self.K, 64) * 64 if self.dtype == "int8" else ceil_div(self.K, 16) * 16
 
 
 F32_BK = (8, 16, 32, 64)
@@ -247,8 +249,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         if splitk != 1:
             raise InvalidConfig("int8 GEMM does not split K across workgroups")
         mfma_k = 32 if mfm == 32 else 64
-        if bk % mfma_k != 0 or view.K % 16 != 0:
+        if bk % mfma_k != 0:
             raise InvalidConfig("BK must be a multiple of the MFMA K extent")
+        if view.K % 16 != 0:
+            raise InvalidConfig("int8 GEMM needs K to be a multiple of 16")
         pad = int(_special(special, "lds_pad")[0]) * 4
         if pad % 16 != 0:
             raise InvalidConfig("int8 LDS padding must be a multiple of 16 bytes")

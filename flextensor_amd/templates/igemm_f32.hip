@@ -30,8 +30,30 @@
 // Within a k-block of 4*KL values, lane group g of an MFMA takes
 // k = 4*g + s at step s for both operands, so the sum over k is unchanged.
 
-#ifndef MODE
-#error "MODE must be defined"
+/* Constants arrive as -DFT_<NAME>=value: single-letter macros on the command line
+ * would be visible to (and break) the runtime-compilation built-in headers. */
+#define MODE FT_MODE
+#define M FT_M
+#define N FT_N
+#define K FT_K
+#define KP FT_KP
+#define MFMA FT_MFMA
+#define WAVES_M FT_WAVES_M
+#define WAVES_N FT_WAVES_N
+#define REP_M FT_REP_M
+#define REP_N FT_REP_N
+#define BK FT_BK
+#define STAGES FT_STAGES
+#define SPLITK FT_SPLITK
+#define GROUP_M FT_GROUP_M
+#define XCD_REMAP FT_XCD_REMAP
+#define APAD FT_APAD
+#define BPAD FT_BPAD
+#define AV FT_AV
+#define BV FT_BV
+
+#ifndef FT_MODE
+#error "FT_MODE must be defined"
 #endif
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -103,6 +125,17 @@ typedef float bvec_t;
 #endif
 
 #if MODE == 1
+#define CB FT_CB
+#define CC FT_CC
+#define CH FT_CH
+#define CW FT_CW
+#define CR FT_CR
+#define CS FT_CS
+#define CSTR FT_CSTR
+#define CPAD FT_CPAD
+#define CDIL FT_CDIL
+#define CP FT_CP
+#define CQ FT_CQ
 /* conv geometry, all compile-time: input [CB][CC][CH][CW], kernel CR x CS,
  * stride CSTR, padding CPAD, dilation CDIL, output CP x CQ. */
 #define OHW (CP * CQ)

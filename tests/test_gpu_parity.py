@@ -1,0 +1,416 @@
+"""Device parity: tuned-kernel plans, called through the C-ABI (libftrocm.so),
+against the CPU oracle on the same seeded inputs.
+
+Acceptance: fp32  max|out - ref| / max|ref| <= 1e-5 ; int32 bit-exact.
+Sizes are chosen so that the oracle finishes in seconds; the five benchmark
+configurations are also covered at full size.
+"""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+if not torch.cuda.is_available():
+    pytest.skip("no GPU visible", allow_module_level=True)
+
+from flextensor_amd import runtime as rt  # noqa: E402
+from flextensor_amd.measure import (Measurer, WrongResult, compare_on_device,  # noqa: E402
+                                    run_default_schedule, seeded_inputs)
+from flextensor_amd.plan import build, current_stream  # noqa: E402
+from flextensor_amd.scheduler import schedule, schedule_with_config  # noqa: E402
+from flextensor_amd.task import (TASK_TABLE, Task, register, gemm, gemm_int8, conv2d,  # noqa: E402
+                                 depthwise_conv2d)
+from flextensor_amd.nn import gemm as op_gemm  # noqa: E402
+from flextensor_amd.te import placeholder  # noqa: E402
+from flextensor_amd.utils import Config, ceil_div  # noqa: E402
+
+TOL = 1e-5
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "small_cases.npz"))
+KEYS = ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]
+
+
+def rel(a, b):
+    b = np.asarray(b, np.float64)
+    return float(np.max(np.abs(np.asarray(a, np.float64) - b)) / np.max(np.abs(b)))
+
+
+def key_of(category, name, args):
+    return Task(category, name, None, args, "rocm", 0).key
+
+
+def gcfg(M, N, K, wm, rm, wn, rn, mf, bk, sk=1, st=2, gm=4, xcd=1):
+    c = {k: [] for k in KEYS}
+    c["spatial"] = [[ceil_div(M, wm * rm * mf), wm, rm, mf], [ceil_div(N, wn * rn * mf), wn, rn, mf]]
+    c["reduce"] = [[sk, K // (sk * bk), bk]]
+    c["unroll"], c["fuse"], c["reorder"] = [[st, 1]], [[gm]], [[xcd]]
+    return c
+
+
+def dcfg(b, c, p, q, th, tw, waves):
+    cfg = {k: [] for k in KEYS}
+    cfg["spatial"] = [[b, 1, 1, 1], [c, 1, 1, 1], [ceil_div(p, th), 1, 1, th], [ceil_div(q, tw), 1, 1, tw]]
+    cfg["fuse"] = [[waves]]
+    return cfg
+
+
+def run_plan(key, configs, host_inputs):
+    """Lower, build through the C-ABI, run once; returns the output as numpy."""
+    s, bufs = schedule_with_config(key, configs)
+    func = build(s, bufs, "rocm")
+    tdt = {"float32": torch.float32, "int32": torch.int32}[bufs[-1].dtype]
+    ins = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in host_inputs]
+    out = torch.full(bufs[-1].shape, -77, dtype=tdt, device="cuda")
+    func(*ins, out)
+    torch.cuda.synchronize()
+    func.close()
+    return out.cpu().numpy()
+
+
+def conv_cfgs(op_cfg, inline=None):
+    g = None
+    if inline is not None:
+        g = {k: [] for k in KEYS}
+        g["inline"] = [inline]
+    return Config([{k: [] for k in KEYS}, op_cfg], g)
+
+
+# ---------------------------------------------------------------- runtime --
+
+def test_device_is_gfx950_and_library_in_tree():
+    p = rt.device_props(0)
+    assert p["arch"].startswith("gfx950") and p["wave_size"] == 64
+    assert p["lds_bytes_per_block"] == 160 * 1024
+    assert os.path.dirname(rt.LIB_PATH).endswith("flextensor_amd")
+
+
+def test_raw_cabi_launch_and_timing():
+    src = ('extern "C" __global__ void axpy(float* y, const float* x, float a, int n)'
+           '{ int i = blockIdx.x * 256 + threadIdx.x; if (i < n) y[i] += a * x[i]; }')
+    mod = rt.Module.from_source(src, "axpy")
+    n = 100003
+    x = torch.arange(n, dtype=torch.float32, device="cuda")
+    y = torch.ones(n, dtype=torch.float32, device="cuda")
+    args = [rt.ptr(y), rt.ptr(x), rt.f32(2.0), rt.i32(n)]
+    mod.launch((ceil_div(n, 256),), (256,), args, stream=current_stream())
+    torch.cuda.synchronize()
+    assert torch.equal(y, 1 + 2 * x)
+    ms = mod.time((ceil_div(n, 256),), (256,), args, warmup=1, iters=3, stream=current_stream())
+    assert 0 < ms < 10
+    assert torch.equal(y, 1 + 2 * 5 * x)  # 1 + 1 + 3 launches in total
+    a = mod.attrs()
+    assert a["private_bytes"] == 0 and a["num_regs"] > 0
+    with pytest.raises(rt.RuntimeError_):
+        rt.Module(b"\x7fELFgarbage" + b"\0" * 64, "axpy")
+    with pytest.raises(rt.RuntimeError_):
+        mod.launch((0,), (256,), args)
+
+
+# ------------------------------------------------------- golden fixtures --
+
+def test_golden_gemm_small_ragged():
+    a, b = GOLD["gemm_a"], GOLD["gemm_b"]       # 37x64 @ 64x29: ragged M and N
+    register(gemm, "gemm", "gemm", (37, 64, 29), "rocm", 0)
+    key = key_of("gemm", "gemm", (37, 64, 29))
+    for cfg in (None, gcfg(37, 29, 64, 1, 1, 1, 1, 16, 16), gcfg(37, 29, 64, 2, 1, 1, 1, 32, 32),
+                gcfg(37, 29, 64, 1, 2, 2, 1, 16, 16, sk=2), gcfg(37, 29, 64, 1, 1, 1, 1, 32, 8, st=1)):
+        out = run_plan(key, Config([cfg] if cfg else [], None), [a, b])
+        assert rel(out, GOLD["gemm_c"]) <= TOL, cfg
+
+
+def test_golden_gemm_int8_small_ragged():
+    a, b = GOLD["i8_a"], GOLD["i8_b"]           # 19x48 · (23x48)^T, K tail, extreme products
+    register(gemm_int8, "gemm", "gemm_int8", (19, 48, 23), "rocm", 0)
+    key = key_of("gemm", "gemm_int8", (19, 48, 23))
+    for cfg in (None, gcfg(19, 23, 64, 1, 1, 1, 1, 16, 64), gcfg(19, 23, 64, 1, 1, 2, 1, 32, 64),
+                gcfg(19, 23, 64, 2, 1, 1, 1, 16, 64, st=1)):
+        out = run_plan(key, Config([cfg] if cfg else [], None), [a, b])
+        assert np.array_equal(out, GOLD["i8_c"]), cfg
+        assert out[0, 0] == 48 * 128 * 128
+
+
+def test_golden_conv_small():
+    x = GOLD["conv_a_x"]                         # [2,5,9,6]; K = 45 -> padded K tail
+    for wname, yname, ks, pad in (("conv_a_w", "conv_a_y", 3, 1), ("conv_b_w", "conv_b_y", 1, 0)):
+        w = GOLD[wname]
+        args = (2, 5, 9, 6, w.shape[0], ks, 1, pad, 1, 1)
+        register(conv2d, "conv2d", "t", args, "rocm", 0)
+        key = key_of("conv2d", "t", args)
+        for inline in (None, [1, 0], [0, 0]):
+            if pad == 0 and inline == [0, 0]:
+                pass  # a zero-width pad kernel is still a valid copy
+            out = run_plan(key, conv_cfgs({}, inline), [x, w])
+            assert rel(out, GOLD[yname]) <= TOL, (wname, inline)
+
+
+def test_golden_depthwise_reference_case():
+    # the reference's own case: x [4,6,7,7], w [6,3,3,3], stride 2, pad 1, dilation 2
+    x, w = GOLD["dw_x"], GOLD["dw_w"]
+    args = (4, 6, 7, 7, 3, 3, 2, 1, 2)
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    for cfg in ({}, dcfg(4, 18, 3, 3, 1, 1, 1), dcfg(4, 18, 3, 3, 2, 2, 2), dcfg(4, 18, 3, 3, 3, 1, 4)):
+        out = run_plan(key, conv_cfgs(cfg), [x, w])
+        assert rel(out, GOLD["dw_y"]) <= TOL, cfg
+    x, w = GOLD["dw1_x"], GOLD["dw1_w"]          # [2,5,8,12], 3x3 s1 p1: vector path
+    args = (2, 5, 8, 12, 1, 3, 1, 1, 1)
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    for cfg in ({}, dcfg(2, 5, 8, 12, 4, 4, 1), dcfg(2, 5, 8, 12, 7, 4, 2), dcfg(2, 5, 8, 12, 2, 2, 1)):
+        for inline in (None, [0, 0]):
+            out = run_plan(key, conv_cfgs(cfg, inline), [x, w])
+            assert rel(out, GOLD["dw1_y"]) <= TOL, (cfg, inline)
+
+
+# ------------------------------------------------ seeded inputs vs oracle --
+
+GEMM_CASES = [
+    # M, K, N, config knobs
+    (256, 256, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16)),
+    (256, 256, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=32, sk=2)),
+    (256, 256, 256, dict(wm=1, rm=4, wn=4, rn=1, mf=16, bk=64, st=1, gm=1, xcd=0)),
+    (200, 136, 328, dict(wm=2, rm=1, wn=1, rn=3, mf=32, bk=8)),      # ragged M, N; N % 4 == 0
+    (96, 80, 67, dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=16)),        # N % 4 != 0 -> scalar loads
+    (512, 1024, 128, dict(wm=4, rm=1, wn=1, rn=2, mf=32, bk=32, sk=8, gm=2)),
+]
+
+
+@pytest.mark.parametrize("M,K,N,kn", GEMM_CASES)
+def test_gemm_f32_vs_oracle(oracle, M, K, N, kn):
+    register(gemm, "gemm", "gemm", (M, K, N), "rocm", 0)
+    key = key_of("gemm", "gemm", (M, K, N))
+    ops, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=M + N)
+    kp = ceil_div(K, 16) * 16
+    out = run_plan(key, Config([gcfg(M, N, kp, **kn)], None), [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+    assert rel(out, oracle.gemm_f32_c(a, b)) <= TOL
+
+
+def test_gemm_transpose_b_vs_oracle(oracle):
+    def wrap(M, K, N):
+        A = placeholder((M, K), name="A")
+        B = placeholder((N, K), name="B")
+        C = op_gemm(A, B, transposeB=True)
+        return [C.op], [A, B, C]
+    register(wrap, "gemm", "gemm_nt", (160, 96, 224), "rocm", 0)
+    key = key_of("gemm", "gemm_nt", (160, 96, 224))
+    _, bufs = wrap(160, 96, 224)
+    a, b = seeded_inputs(bufs, seed=9)
+    for cfg in (None, gcfg(160, 224, 96, 2, 1, 2, 1, 32, 16), gcfg(160, 224, 96, 1, 2, 2, 2, 16, 32, sk=3)):
+        out = run_plan(key, Config([cfg] if cfg else [], None), [a, b])
+        assert rel(out, oracle.gemm_f32_c(a, b, transB=True)) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N,kn", [
+    (256, 256, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=64)),
+    (256, 512, 384, dict(wm=1, rm=4, wn=2, rn=2, mf=16, bk=128, st=1)),
+    (136, 208, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64)),      # ragged everywhere, K tail
+    (512, 256, 512, dict(wm=2, rm=4, wn=2, rn=4, mf=32, bk=128, gm=2, xcd=0)),
+])
+def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
+    register(gemm_int8, "gemm", "gemm_int8", (M, K, N), "rocm", 0)
+    key = key_of("gemm", "gemm_int8", (M, K, N))
+    _, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=K)
+    assert a.min() == -128 and a.max() == 127
+    out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], None), [a, b])
+    assert np.array_equal(out, oracle.gemm_i8_c(a, b))
+    assert np.array_equal(out, oracle.gemm_i8_np(a, b))
+
+
+CONV_CASES = [
+    # batch, C, H, W, K, k, stride, pad, dil, knobs
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=16)),
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=16, sk=3)),
+    ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16)),   # stride 2, K=72 -> 80
+    ((3, 6, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32)),   # dilation 2
+    ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=32)),    # 1x1, N=392
+    ((1, 3, 32, 32, 16, 7, 2, 3, 1, 1), dict(wm=1, rm=1, wn=4, rn=1, mf=16, bk=16)),   # 7x7 s2 p3, K=147
+]
+
+
+@pytest.mark.parametrize("args,kn", CONV_CASES)
+def test_conv2d_vs_oracle(oracle, args, kn):
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    key = key_of("conv2d", "t", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
+    assert ref.shape == bufs[-1].shape
+    M, N, K = ko, nb * ref.shape[2] * ref.shape[3], c * ks * ks
+    cfg = gcfg(M, N, ceil_div(K, 16) * 16, **kn)
+    for inline in ([1, 0], [0, 0]):
+        out = run_plan(key, conv_cfgs(cfg, inline), [x, w])
+        assert rel(out, ref) <= TOL, inline
+        assert rel(out, oracle.conv2d_nchw_np(x, w, st, pd, dl, g)) <= TOL
+
+
+@pytest.mark.parametrize("args,th,tw,waves", [
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 4, 4, 4),
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 7, 4, 1),
+    ((1, 8, 15, 13, 2, 3, 1, 1, 1), 4, 4, 2),      # odd plane, factor 2
+    ((1, 8, 15, 13, 2, 3, 2, 1, 1), 2, 2, 1),      # stride 2
+    ((2, 4, 9, 9, 1, 5, 1, 2, 1), 1, 4, 1),        # 5x5
+])
+def test_depthwise_vs_oracle(oracle, args, th, tw, waves):
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, f, ks, st, pd, dl = args
+    ref = oracle.depthwise_nchw_c(x, w, st, pd, dl)
+    b_, co, p, q = ref.shape
+    out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves)), [x, w])
+    assert rel(out, ref) <= TOL
+
+
+def test_default_schedule_kernels_vs_oracle(oracle):
+    """The plain kernels every candidate is gated against are themselves right."""
+    s = current_stream()
+    for args in [(2, 6, 9, 11, 9, 3, 2, 1, 2, 3), (1, 4, 8, 8, 6, 3, 1, 1, 1, 1)]:
+        ops, bufs = conv2d(*args)
+        x, w = seeded_inputs(bufs, 1)
+        out = torch.empty(bufs[-1].shape, device="cuda")
+        run_default_schedule(ops, [torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), out], s)
+        ref = oracle.conv2d_nchw_c(x, w, args[6], args[7], args[8], args[9])
+        assert rel(out.cpu().numpy(), ref) <= 1e-6
+    ops, bufs = depthwise_conv2d(2, 6, 9, 11, 3, 3, 2, 1, 2)
+    x, w = seeded_inputs(bufs, 2)
+    out = torch.empty(bufs[-1].shape, device="cuda")
+    run_default_schedule(ops, [torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), out], s)
+    assert rel(out.cpu().numpy(), oracle.depthwise_nchw_c(x, w, 2, 1, 2)) <= 1e-6
+    ops, bufs = gemm(70, 50, 90)
+    a, b = seeded_inputs(bufs, 3)
+    out = torch.empty(bufs[-1].shape, device="cuda")
+    run_default_schedule(ops, [torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), out], s)
+    assert rel(out.cpu().numpy(), oracle.gemm_f32_c(a, b)) <= 1e-6
+    ops, bufs = gemm_int8(70, 64, 90)
+    a, b = seeded_inputs(bufs, 4)
+    out = torch.empty(bufs[-1].shape, dtype=torch.int32, device="cuda")
+    run_default_schedule(ops, [torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), out], s)
+    assert np.array_equal(out.cpu().numpy(), oracle.gemm_i8_c(a, b))
+
+
+# ------------------------------------------- the five benchmark configs ---
+
+FULL = {
+    "gemm": "gemm_gemm_(1024, 1024, 1024)_rocm(0)",
+    "conv2": "conv2d_baseline0_(1, 64, 56, 56, 64, 3, 1, 1, 1, 1)_rocm(0)",
+    "conv3a": "conv2d_baseline1_(8, 256, 14, 14, 512, 3, 1, 1, 1, 1)_rocm(0)",
+    "conv3b": "conv2d_baseline2_(8, 512, 7, 7, 2048, 1, 1, 0, 1, 1)_rocm(0)",
+    "dw": "conv2d_depthwise_(8, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)",
+    "i8": "gemm_gemm_int8_(4096, 4096, 4096)_rocm(0)",
+}
+
+
+def tuned_configs(key):
+    from flextensor_amd.tuned import lookup
+    cfg = lookup(key)
+    return cfg if cfg is not None else Config([], None)
+
+
+def test_full_size_gemm_fp32(oracle):
+    key = FULL["gemm"]
+    _, bufs = TASK_TABLE[key].func(*TASK_TABLE[key].args)
+    a, b = seeded_inputs(bufs, 0)
+    out = run_plan(key, tuned_configs(key), [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+    rows = oracle.gemm_f32_c(a[:48], b)           # fp32 sequential-k oracle on a row sample
+    assert rel(out[:48], rows) <= TOL
+
+
+@pytest.mark.parametrize("name", ["conv2", "conv3a", "conv3b"])
+def test_full_size_conv2d(oracle, name):
+    key = FULL[name]
+    args = TASK_TABLE[key].args
+    _, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, 0)
+    out = run_plan(key, tuned_configs(key), [x, w])
+    ref = oracle.conv2d_nchw_c(x, w, args[6], args[7], args[8], args[9])
+    assert rel(out, ref) <= TOL
+    assert rel(out, oracle.conv2d_nchw_np(x, w, args[6], args[7], args[8], args[9])) <= TOL
+
+
+def test_full_size_depthwise(oracle):
+    key = FULL["dw"]
+    args = TASK_TABLE[key].args
+    _, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, 0)
+    out = run_plan(key, tuned_configs(key), [x, w])
+    assert rel(out, oracle.depthwise_nchw_c(x, w, 1, 1, 1)) <= TOL
+    # linearity in the input, a size-independent property
+    x2 = np.random.default_rng(5).uniform(-1, 1, x.shape).astype(np.float32)
+    o2 = run_plan(key, tuned_configs(key), [x2, w])
+    o12 = run_plan(key, tuned_configs(key), [x + x2, w])
+    assert rel(o12, out.astype(np.float64) + o2) <= TOL
+
+
+def test_full_size_gemm_int8_bit_exact(oracle):
+    key = FULL["i8"]
+    _, bufs = TASK_TABLE[key].func(*TASK_TABLE[key].args)
+    a, b = seeded_inputs(bufs, 0)
+    out = run_plan(key, tuned_configs(key), [a, b])
+    assert np.array_equal(out, oracle.gemm_i8_np(a, b))              # exact, float64 BLAS
+    assert np.array_equal(out[100:132], oracle.gemm_i8_c(a, b, 100, 132)[100:132])
+    # size-independent properties: worst-case magnitude and a permutation operand
+    a2 = np.full_like(a, -128)
+    out2 = run_plan(key, tuned_configs(key), [a2, a2])
+    assert out2.min() == out2.max() == 4096 * 128 * 128              # 2^26, no overflow
+    eye = np.eye(4096, dtype=np.int8)
+    out3 = run_plan(key, tuned_configs(key), [a, eye])
+    assert np.array_equal(out3, a.astype(np.int32))                  # A · Iᵀ = A
+    out4 = run_plan(key, tuned_configs(key), [a, b])
+    assert np.array_equal(out4, out)                                 # deterministic
+
+
+# --------------------------------------------------- measure / search path --
+
+def test_correctness_gate_rejects_wrong_output():
+    key = "gemm_gemm_(256, 256, 256)_rocm(0)"
+    m = Measurer(key)
+    s, _ = schedule_with_config(key, Config([], None))
+    ms = m.evaluate(s, number=3)
+    assert 0 < ms < 10
+    ok, metric = m.check(m.sets[0][-1])
+    assert ok and metric <= TOL
+    m.ref += 1.0                                   # corrupt the default-schedule result
+    with pytest.raises(WrongResult):
+        m.evaluate(s, number=1)
+    bad = m.sets[0][-1].clone()
+    bad[3, 5] = float("nan")
+    assert compare_on_device(bad, m.sets[0][-1], current_stream())[0] is False
+
+
+def test_builtplan_rejects_mismatched_tensors():
+    key = "gemm_gemm_(256, 256, 256)_rocm(0)"
+    s, bufs = schedule_with_config(key, Config([], None))
+    f = build(s, bufs, "rocm")
+    a = torch.zeros(256, 256, device="cuda")
+    with pytest.raises(ValueError):
+        f(a, a)
+    with pytest.raises(ValueError):
+        f(a, a, torch.zeros(256, 128, device="cuda"))
+    with pytest.raises(ValueError):
+        f(a, a, torch.zeros(256, 256, device="cuda", dtype=torch.int32))
+    with pytest.raises(ValueError):
+        f(a, a.t(), torch.zeros(256, 256, device="cuda")) if not a.t().is_contiguous() else None
+    with pytest.raises(ValueError):
+        f(a.cpu(), a, a)
+    f.close()
+
+
+def test_schedule_on_device_small_gemm(oracle):
+    """End to end: search a few points on the GPU, replay the winner, check it."""
+    np.random.seed(0)
+    key = "gemm_gemm_(512, 256, 512)_rocm(0)"
+    s, bufs, configs = schedule(key, op_trial=2, graph_trial=1, op_stop=2, parallel=8, number=5,
+                                timeout=20, warm_up=(1, 8), verbose=False)
+    a, b = seeded_inputs(bufs, 11)
+    out = run_plan(key, configs, [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+    s2, _ = schedule_with_config(key, Config(*__import__("json").loads(__import__("json").dumps(configs))))
+    assert s2.describe() == s.describe()

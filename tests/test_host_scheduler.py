@@ -1,0 +1,244 @@
+"""Task registry, search driver with a host-side cost function, config replay,
+lowering invariants and error behaviour. No GPU."""
+import json
+import math
+
+import numpy as np
+import pytest
+
+from flextensor_amd import scheduler as sch
+from flextensor_amd.model import WalkerGroup
+from flextensor_amd.scheduler import flatten_graph, schedule, schedule_with_config
+from flextensor_amd.space import generate_space_intra_op
+from flextensor_amd.task import TASK_TABLE, Task, register_task, gemm, conv2d
+from flextensor_amd.templates import gfx950
+from flextensor_amd.utils import Config
+
+GEMM = "gemm_gemm_(1024, 1024, 1024)_rocm(0)"
+CONV = "conv2d_baseline0_(1, 64, 56, 56, 64, 3, 1, 1, 1, 1)_rocm(0)"
+DW = "conv2d_depthwise_(8, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)"
+I8 = "gemm_gemm_int8_(4096, 4096, 4096)_rocm(0)"
+CONV1x1 = "conv2d_baseline2_(8, 512, 7, 7, 2048, 1, 1, 0, 1, 1)_rocm(0)"
+
+
+def test_task_key_format_and_registry():
+    # key format of the reference: "{category}_{name}_{args}_{target}({dev})"
+    t = Task("gemm", "gemm", None, (1024, 1024, 1024), "llvm", 0)
+    assert t.key == "gemm_gemm_(1024, 1024, 1024)_llvm(0)"
+    for k in (GEMM, CONV, DW, I8, CONV1x1):
+        assert k in TASK_TABLE
+    for dev in range(4):
+        assert "gemm_gemm_(1024, 1024, 1024)_rocm(%d)" % dev in TASK_TABLE
+    with pytest.raises(KeyError):
+        schedule("gemm_gemm_(3, 3, 3)_rocm(0)")
+    with pytest.raises(RuntimeError):
+        t.set_specific_space("x", "range", [1, 2])
+    # drivers build a func=None task for the key and look the real one up
+    probe = Task("conv2d", "baseline0", None, (1, 64, 56, 56, 64, 3, 1, 1, 1, 1), "rocm", 0)
+    ops, bufs = TASK_TABLE[probe.key].func(*TASK_TABLE[probe.key].args)
+    assert [b.shape for b in bufs] == [(1, 64, 56, 56), (64, 64, 3, 3), (1, 64, 56, 56)]
+    ops, bufs = TASK_TABLE[I8].func(*TASK_TABLE[I8].args)
+    assert [b.dtype for b in bufs] == ["int8", "int8", "int32"]
+    # no override unless asked
+    other = Task("gemm", "gemm", lambda *a: None, (1024, 1024, 1024), "rocm", 0)
+    register_task(other)
+    assert TASK_TABLE[GEMM].func is gemm
+    assert "lds_pad" in TASK_TABLE[GEMM].special_space
+
+
+def test_unsupported_target_and_method():
+    register_task(Task("gemm", "gemm", gemm, (64, 64, 64), "cuda", 0), override=True)
+    with pytest.raises(RuntimeError, match="no support for target"):
+        schedule("gemm_gemm_(64, 64, 64)_cuda(0)")
+    with pytest.raises(RuntimeError, match="no support for target"):
+        schedule_with_config("gemm_gemm_(64, 64, 64)_cuda(0)", Config([], None))
+    with pytest.raises(RuntimeError, match="no support for method"):
+        schedule(GEMM, method="annealing", evaluator=lambda *a: 1.0)
+
+
+def test_default_lowering_of_baseline_tasks():
+    for key in (GEMM, CONV, DW, I8, CONV1x1):
+        s, bufs = schedule_with_config(key, Config([], None))
+        assert len(bufs) == 3 and s.specs
+        main = s.specs[-1]
+        assert main.block[0] % 64 == 0 and main.block[0] <= 1024
+        for spec in s.specs:
+            assert all(g >= 1 for g in spec.grid)
+    s, _ = schedule_with_config(CONV, Config([], None))
+    d = s.specs[-1].defines
+    assert d["MODE"] == 1 and (d["M"], d["N"], d["K"]) == (64, 3136, 576) and d["CPAD"] == 1
+    assert [a[1] for a in s.specs[-1].args] == ["in1", "in0", "out"]  # A = weight, B = image
+    assert s.intermediates == {}
+
+
+def test_graph_config_not_inlined_materialises_padding():
+    empty = {k: [] for k in ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]}
+    g = dict(empty)
+    g["inline"] = [[0, 0]]
+    s, _ = schedule_with_config(CONV, Config([dict(empty), {}], g))
+    assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "igemm_f32"]
+    assert s.intermediates == {"tmp0": ((1, 64, 58, 58), "float32")}
+    d = s.specs[-1].defines
+    assert d["CPAD"] == 0 and d["CH"] == 58 and d["CW"] == 58
+    assert [a[1] for a in s.specs[-1].args] == ["in1", "tmp0", "out"]
+    g["inline"] = [[1, 1]]
+    with pytest.raises(ValueError):
+        schedule_with_config(CONV, Config([dict(empty), {}], g))
+
+
+def _gemm_cfg(sp0, sp1, red, stages=2, gm=4, xcd=1):
+    c = {k: [] for k in ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]}
+    c.update(spatial=[sp0, sp1], reduce=[red], unroll=[[stages, 1]], fuse=[[gm]], reorder=[[xcd]])
+    return c
+
+
+def test_lowering_rejects_bad_configs():
+    ok = _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16])
+    s, _ = schedule_with_config(GEMM, Config([ok], None))
+    d = s.specs[0].defines
+    assert (d["WAVES_M"], d["REP_M"], d["MFMA"], d["BK"], d["SPLITK"]) == (2, 1, 32, 16, 1)
+    assert s.specs[0].grid == (256, 1, 1) and s.specs[0].block == (256, 1, 1)
+    bad = [
+        _gemm_cfg([16, 2, 1, 32], [32, 2, 1, 16], [1, 64, 16]),   # mixed MFMA edge
+        _gemm_cfg([15, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16]),   # wrong grid level
+        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 8]),    # K product != K
+        _gemm_cfg([2, 2, 8, 32], [2, 2, 8, 32], [1, 64, 16]),     # 1024 accumulators
+        _gemm_cfg([8, 8, 1, 16], [8, 8, 1, 16], [1, 64, 16]),     # 64 wavefronts
+        _gemm_cfg([32, 2, 1, 16], [32, 2, 1, 16], [1, 128, 8]),   # BK < 16 with 16x16x4
+        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=3),
+    ]
+    for cfg in bad:
+        with pytest.raises(gfx950.InvalidConfig):
+            schedule_with_config(GEMM, Config([cfg], None))
+    # split-K adds the zero-fill kernel and multiplies the grid
+    s, _ = schedule_with_config(GEMM, Config([_gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [2, 32, 16])], None))
+    assert [x.kernel for x in s.specs] == ["fill_zero_f32", "igemm_f32"] and s.specs[1].grid[0] == 512
+    # int8 never splits K
+    i8 = _gemm_cfg([16, 2, 4, 32], [16, 2, 4, 32], [2, 32, 64])
+    with pytest.raises((gfx950.InvalidConfig, AssertionError)):
+        schedule_with_config(I8, Config([i8], None))
+
+
+def test_lds_budget_respected_over_whole_space():
+    ops, _ = TASK_TABLE[I8].func(*TASK_TABLE[I8].args)
+    op_lst, down = flatten_graph(ops)
+    space = generate_space_intra_op(op_lst[0], down, target="rocm")
+    wg = WalkerGroup("t", space)
+    rng = np.random.default_rng(0)
+    n_ok = 0
+    for _ in range(300):
+        idx = {name: int(rng.integers(0, len(sub))) for name, sub in space.items()}
+        cfg = wg.to_config(idx)
+        try:
+            s, _ = schedule_with_config(I8, Config([cfg], None))
+        except gfx950.InvalidConfig:
+            continue
+        n_ok += 1
+        d = s.specs[-1].defines
+        bm = d["WAVES_M"] * d["REP_M"] * d["MFMA"]
+        bn = d["WAVES_N"] * d["REP_N"] * d["MFMA"]
+        assert d["STAGES"] * (bm + bn) * (d["BK"] + d["PAD"]) <= 160 * 1024
+        assert d["REP_M"] * d["REP_N"] * d["MFMA"] ** 2 // 64 <= 256
+    assert n_ok > 20
+
+
+def _synthetic_cost(task_key, cfg, op_pos, number):
+    """Smooth host-side cost with a known optimum, defined on the lowered kernel."""
+    s, _ = schedule_with_config(task_key, cfg, op_pos=op_pos)
+    d = s.specs[-1].defines
+    bm = d["WAVES_M"] * d["REP_M"] * d["MFMA"]
+    bn = d["WAVES_N"] * d["REP_N"] * d["MFMA"]
+    cost = abs(math.log2(bm) - 6) + abs(math.log2(bn) - 6) + abs(math.log2(d["BK"]) - 5)
+    cost += 0.5 * (d["SPLITK"] - 1) + 0.25 * (d["STAGES"] != 2) + 0.1 * abs(d["GROUP_M"] - 4)
+    cost += 0.3 * (d["MFMA"] != 32) + 0.2 * (d["WAVES_M"] * d["WAVES_N"] != 4)
+    return 1.0 + cost
+
+
+def test_schedule_searching_finds_known_optimum_and_roundtrips():
+    np.random.seed(0)
+    s, bufs, configs = schedule(GEMM, op_trial=30, op_stop=30, graph_trial=2, parallel=4,
+                                evaluator=_synthetic_cost, warm_up=(3, 10), verbose=False)
+    best = _synthetic_cost(GEMM, configs, None, 1)
+    assert best <= 1.5, best
+    assert isinstance(configs, Config) and len(configs.op_config_lst) == 1
+    assert sorted(configs.op_config_lst[0]) == sorted(
+        ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"])
+    assert len(configs.graph_config["special"]) == len(TASK_TABLE[GEMM].special_space)
+    # JSON log line round trip (the reference's `key:json` format)
+    line = GEMM + ":" + json.dumps(configs)
+    name, string = line.split(":", 1)
+    obj = json.loads(string)
+    s2, _ = schedule_with_config(name, Config(obj[0], obj[1]))
+    assert s2.describe() == s.describe()
+
+
+def test_schedule_random_method_and_conv_graph():
+    np.random.seed(1)
+    calls = []
+
+    def cost(task_key, cfg, op_pos, number):
+        calls.append(op_pos)
+        s, _ = schedule_with_config(task_key, cfg, op_pos=op_pos)
+        return 1.0 + 0.01 * len(s.specs) + 1e-4 * s.specs[-1].grid[0]
+
+    s, bufs, configs = schedule(CONV, op_trial=3, graph_trial=2, parallel=3, method="random",
+                                evaluator=cost, verbose=False)
+    assert len(configs.op_config_lst) == 2          # [Padding, conv]
+    assert not any(configs.op_config_lst[0].values())  # padding has no knobs
+    assert configs.graph_config["inline"][0] == [1, 0]  # fused padding is cheaper here
+    assert 1 in calls and None in calls
+
+
+def test_failing_candidates_become_inf_and_search_survives():
+    np.random.seed(2)
+    n = {"calls": 0}
+
+    def flaky(task_key, cfg, op_pos, number):
+        n["calls"] += 1
+        if n["calls"] % 3 == 0:
+            raise RuntimeError("candidate crashed")
+        return _synthetic_cost(task_key, cfg, op_pos, number)
+
+    s, bufs, configs = schedule(GEMM, op_trial=5, graph_trial=1, parallel=2, evaluator=flaky,
+                                warm_up=(2, 6), verbose=False)
+    assert configs.op_config_lst[0]["spatial"]
+
+
+def test_all_invalid_warm_up_escalates_then_gives_up():
+    def never(task_key, cfg, op_pos, number):
+        raise RuntimeError("nothing builds")
+
+    ops, _ = TASK_TABLE[GEMM].func(*TASK_TABLE[GEMM].args)
+    op_lst, down = flatten_graph(ops)
+    space = generate_space_intra_op(op_lst[0], down, target="rocm")
+    o = sch.OpScheduler(GEMM, 0, space, parallel=2, timeout=1, evaluator=never)
+    o.verbose = False
+    o._warm_up(1, 4, Config([], None), ["fuse", "reorder", "spatial", "reduce", "unroll"], max_repeat=3)
+    assert o.walker_group.top1() == {} and o.timeout == 1
+
+
+def test_walker_group_heap_semantics():
+    ops, _ = gemm(256, 256, 256)
+    op_lst, down = flatten_graph(ops)
+    space = generate_space_intra_op(op_lst[0], down, target="rocm")
+    wg = WalkerGroup("g", space)
+    pts = []
+    np.random.seed(3)
+    ret = wg.forward(5)
+    for i in range(5):
+        idx = {name: int(ret[name][1][i]) for name in ret}
+        pts.append(idx)
+        wg.record(idx, float(5 - i))
+    assert wg.top1_value() == 1.0 and wg.top1() == pts[4]
+    assert [v for _, v in wg.topk(3, with_value=True)] == [1.0, 2.0, 3.0] and wg.mem_size == 5
+    assert wg.ever_met(pts[0]) and wg.pop_top().value == 1.0 and wg.mem_size == 4
+    nxt, acts = wg.full_walk(pts[0], no_repeat=True)
+    assert all(not wg.ever_met(n) for n in nxt) and len(nxt) == len(acts)
+    for n_, (name, d) in zip(nxt, acts):
+        diff = [k for k in n_ if n_[k] != pts[0][k]]
+        assert diff == [name]
+    cfg = wg.to_config(pts[0])
+    assert len(cfg["spatial"]) == 2 and len(cfg["reduce"]) == 1 and cfg["inline"] == []
+    # a hopeless value is (almost surely) rejected by the Boltzmann filter
+    wg.record(nxt[0], 1e9, random_reject=True)
+    assert wg.mem_size == 4 and wg.ever_met(nxt[0])

@@ -1,0 +1,186 @@
+"""Pins the CPU oracle (oracle/oracle.c) against independent routines.
+
+Each check is chosen so that a plausible mistake fails it: a transposed
+operand (non-square GEMM), a swapped rh/rw (non-square kernels and images),
+wrong group or factor indexing (groups=3, factor=3), a wrong padding or
+dilation sign (stride 2, pad 1, dilation 2 — the reference's own test case,
+flextensor/test/test_ops.py:85-115, 152-184), int8 sign handling (-128 * -128).
+"""
+import os
+
+import numpy as np
+import pytest
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "small_cases.npz")
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLD)
+
+
+def rel(a, b):
+    return float(np.max(np.abs(np.asarray(a, np.float64) - b)) / np.max(np.abs(b)))
+
+
+def test_out_size_closed_form(oracle):
+    # (in + 2p - d(k-1) - 1)//s + 1, spot values worked by hand
+    assert oracle.lib().ft_conv_out_size(56, 1, 1, 3, 1) == 56
+    assert oracle.lib().ft_conv_out_size(7, 1, 2, 3, 2) == 3
+    assert oracle.lib().ft_conv_out_size(448, 3, 1, 7, 2) == 224
+    assert oracle.lib().ft_conv_out_size(7, 0, 1, 1, 1) == 7
+    for n in range(1, 20):
+        for k in (1, 3, 5):
+            for s in (1, 2, 3):
+                for p in (0, 1, 2):
+                    for d in (1, 2):
+                        if n + 2 * p - d * (k - 1) - 1 < 0:
+                            continue
+                        # count valid window positions by brute force
+                        cnt = len([o for o in range(0, n + 2 * p) if o % s == 0
+                                   and o + d * (k - 1) <= n + 2 * p - 1])
+                        assert oracle.conv_out_size(n, p, d, k, s) == cnt
+                        assert oracle.lib().ft_conv_out_size(n, p, d, k, s) == cnt
+
+
+def test_zero_pad2d_closed_form(oracle):
+    x = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5) + 1
+    p = oracle.zero_pad2d_c(x, (1, 2, 3, 0))
+    assert p.shape == (2, 3, 7, 8)
+    assert np.array_equal(p, oracle.zero_pad2d_np(x, (1, 2, 3, 0)))
+    assert np.array_equal(p[:, :, 1:5, 3:8], x)
+    assert p.sum() == x.sum()
+    assert np.all(p[:, :, 0, :] == 0) and np.all(p[:, :, 5:, :] == 0) and np.all(p[:, :, :, :3] == 0)
+
+
+def test_conv2d_reference_case_golden(oracle, gold):
+    y = oracle.conv2d_nchw_c(gold["conv_g3_x"], gold["conv_g3_w"], 2, 1, 2, 3)
+    assert y.shape == (4, 9, 3, 3)
+    assert rel(y, gold["conv_g3_y"]) < 1e-6
+    y0 = oracle.conv2d_nchw_c(gold["conv_g3_x"], gold["conv_g3_w"], 2, 1, 2, 3, fma=False)
+    assert rel(y0, gold["conv_g3_y"]) < 1e-6
+
+
+def test_conv2d_golden_and_numpy(oracle, gold):
+    x = gold["conv_a_x"]
+    assert rel(oracle.conv2d_nchw_c(x, gold["conv_a_w"], 1, 1, 1, 1), gold["conv_a_y"]) < 1e-6
+    assert rel(oracle.conv2d_nchw_c(x, gold["conv_b_w"], 1, 0, 1, 1), gold["conv_b_y"]) < 1e-6
+    assert rel(oracle.conv2d_nchw_np(x, gold["conv_a_w"], 1, 1, 1, 1), gold["conv_a_y"]) < 1e-12
+    assert rel(oracle.conv2d_nchw_np(gold["conv_g3_x"], gold["conv_g3_w"], 2, 1, 2, 3),
+               gold["conv_g3_y"]) < 1e-12
+
+
+def test_conv2d_vs_torch(oracle):
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    rng = np.random.default_rng(1)
+    for (n, c, h, w, k, r, s_, st, p, d, g) in [
+            (4, 6, 7, 7, 9, 3, 3, 2, 1, 2, 3),     # the reference's case
+            (1, 8, 12, 10, 6, 3, 3, 1, 1, 1, 1),
+            (2, 4, 9, 9, 8, 1, 1, 1, 0, 1, 1),
+            (1, 3, 17, 13, 5, 5, 5, 2, 2, 1, 1),
+            (2, 8, 8, 8, 8, 3, 3, 1, 1, 1, 4)]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (k, c // g, r, s_)).astype(np.float32)
+        ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(), None, st, p, d, g).numpy()
+        assert rel(oracle.conv2d_nchw_c(x, wt, st, p, d, g), ref) < 1e-6
+        assert rel(oracle.conv2d_nchw_np(x, wt, st, p, d, g), ref) < 1e-12
+
+
+def test_conv2d_linearity_and_delta(oracle):
+    rng = np.random.default_rng(2)
+    x1 = rng.uniform(-1, 1, (1, 3, 6, 6)).astype(np.float32)
+    x2 = rng.uniform(-1, 1, (1, 3, 6, 6)).astype(np.float32)
+    w = rng.uniform(-1, 1, (4, 3, 3, 3)).astype(np.float32)
+    y = oracle.conv2d_nchw_np(x1 + x2, w, 1, 1, 1, 1)
+    assert np.allclose(y, oracle.conv2d_nchw_np(x1, w, 1, 1, 1, 1) + oracle.conv2d_nchw_np(x2, w, 1, 1, 1, 1))
+    # a one-hot centre tap copies channel sums: identifies rh/rw/c indexing
+    w = np.zeros((2, 3, 3, 3), np.float32)
+    w[0, 1, 1, 1] = 1.0   # out 0 <- in channel 1, centre
+    w[1, 2, 0, 2] = 1.0   # out 1 <- in channel 2, tap (rh=0, rw=2): shift up 1, left... right 1
+    y = oracle.conv2d_nchw_c(x1, w, 1, 1, 1, 1)
+    assert np.array_equal(y[0, 0], x1[0, 1])
+    exp = np.zeros((6, 6), np.float32)
+    exp[1:, :5] = x1[0, 2][:5, 1:]
+    assert np.array_equal(y[0, 1], exp)
+
+
+def test_depthwise_reference_case_golden(oracle, gold):
+    y = oracle.depthwise_nchw_c(gold["dw_x"], gold["dw_w"], 2, 1, 2)
+    assert y.shape == (4, 18, 3, 3)
+    assert rel(y, gold["dw_y"]) < 1e-6
+    assert rel(oracle.depthwise_nchw_np(gold["dw_x"], gold["dw_w"], 2, 1, 2), gold["dw_y"]) < 1e-12
+    assert rel(oracle.depthwise_nchw_c(gold["dw1_x"], gold["dw1_w"], 1, 1, 1), gold["dw1_y"]) < 1e-6
+
+
+def test_depthwise_vs_torch(oracle):
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    rng = np.random.default_rng(3)
+    for (n, c, h, w, f, k, st, p, d) in [(4, 6, 7, 7, 3, 3, 2, 1, 2), (2, 8, 28, 28, 1, 3, 1, 1, 1),
+                                         (1, 5, 9, 11, 2, 3, 1, 0, 1)]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (c, f, k, k)).astype(np.float32)
+        # weight reshape of the reference's test: [C, f, k, k] -> [C*f, 1, k, k], groups=C
+        ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt.reshape(c * f, 1, k, k)).double(),
+                       None, st, p, d, c).numpy()
+        assert rel(oracle.depthwise_nchw_c(x, wt, st, p, d), ref) < 1e-6
+        assert rel(oracle.depthwise_nchw_np(x, wt, st, p, d), ref) < 1e-12
+
+
+def test_gemm_f32(oracle, gold):
+    a, b = gold["gemm_a"], gold["gemm_b"]
+    assert rel(oracle.gemm_f32_c(a, b), gold["gemm_c"]) < 1e-6
+    assert rel(oracle.gemm_f32_c(a, b, fma=False), gold["gemm_c"]) < 1e-6
+    assert rel(oracle.gemm_f32_c(a, np.ascontiguousarray(b.T), transB=True), gold["gemm_c"]) < 1e-6
+    assert rel(oracle.gemm_np(a, b), gold["gemm_c"]) < 1e-13
+    # identity and a permutation matrix: exact
+    eye = np.eye(64, dtype=np.float32)
+    assert np.array_equal(oracle.gemm_f32_c(a, eye), a)
+    perm = eye[:, ::-1].copy()
+    assert np.array_equal(oracle.gemm_f32_c(a, perm), a[:, ::-1])
+
+
+def test_gemm_i8_exact(oracle, gold):
+    a, b = gold["i8_a"], gold["i8_b"]
+    c = oracle.gemm_i8_c(a, b)
+    assert np.array_equal(c, gold["i8_c"])
+    assert c[0, 0] == 48 * 128 * 128
+    assert np.array_equal(oracle.gemm_i8_np(a, b), gold["i8_c"])
+    # the reference's own check: np.dot(a.astype(int32), b.T.astype(int32))
+    rng = np.random.default_rng(4)
+    a = rng.integers(-128, 127, (40, 96), dtype=np.int8)
+    b = rng.integers(-128, 127, (24, 96), dtype=np.int8)
+    assert np.array_equal(oracle.gemm_i8_c(a, b), np.dot(a.astype("int32"), b.T.astype("int32")))
+    part = oracle.gemm_i8_c(a, b, 8, 16)
+    assert np.array_equal(part[8:16], np.dot(a.astype("int32"), b.T.astype("int32"))[8:16])
+    assert not part[:8].any() and not part[16:].any()
+
+
+def test_cpu_baseline_matches_oracle(oracle):
+    rng = np.random.default_rng(5)
+    a = rng.uniform(-1, 1, (70, 96)).astype(np.float32)
+    b = rng.uniform(-1, 1, (96, 50)).astype(np.float32)
+    c = np.empty((70, 50), np.float32)
+    oracle.baseline_gemm_f32(a, b, c, 32)
+    assert rel(c, oracle.gemm_np(a, b)) < 1e-6
+    x = rng.uniform(-1, 1, (2, 6, 9, 20)).astype(np.float32)
+    w = rng.uniform(-1, 1, (7, 6, 3, 3)).astype(np.float32)
+    for st, p, d in [(1, 1, 1), (2, 1, 1), (1, 2, 2)]:
+        ref = oracle.conv2d_nchw_np(x, w, st, p, d, 1)
+        out = np.empty(ref.shape, np.float32)
+        scratch = np.empty((2, 6, 9 + 2 * p, 20 + 2 * p), np.float32)
+        oracle.baseline_conv2d(x, w, out, scratch, st, p, d)
+        assert rel(out, ref) < 1e-6
+    wd = rng.uniform(-1, 1, (6, 2, 3, 3)).astype(np.float32)
+    for st, p, d in [(1, 1, 1), (2, 1, 2)]:
+        ref = oracle.depthwise_nchw_np(x, wd, st, p, d)
+        out = np.empty(ref.shape, np.float32)
+        scratch = np.empty((2, 6, 9 + 2 * p, 20 + 2 * p), np.float32)
+        oracle.baseline_depthwise(x, wd, out, scratch, st, p, d)
+        assert rel(out, ref) < 1e-6
+    ai = rng.integers(-128, 128, (20, 64), dtype=np.int8)
+    bi = rng.integers(-128, 128, (12, 64), dtype=np.int8)
+    ci = np.zeros((20, 12), np.int32)
+    oracle.baseline_gemm_i8(ai, bi, ci)
+    assert np.array_equal(ci, oracle.gemm_i8_np(ai, bi))

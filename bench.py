@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the tuned hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-headline]
+                    [--workload NAME]
 
 One step = one run of the tuned kernel plan of the headline workload
 (conv2d NCHW fp32, N=1, C=64, H=W=56, K=64, 3x3, stride 1, pad 1) over
@@ -134,6 +135,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
+    ap.add_argument("--workload", default=None, choices=[w[0] for w in WORKLOADS],
+                    help="time this configuration as the headline instead of configs[1] "
+                         "(used to profile one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the tuned kernels are single-device and nothing "
@@ -149,7 +153,10 @@ def main():
     torch.cuda.set_device(0)
     props = rt.device_props(0)
 
-    name, key, ops, nbytes, bound, dtype = WORKLOADS[HEADLINE]
+    headline = HEADLINE if args.workload is None else [w[0] for w in WORKLOADS].index(args.workload)
+    name, key, ops, nbytes, bound, dtype = WORKLOADS[headline]
+    if dtype == "i8":
+        args.steps = min(args.steps, 500)
     built, m, plan = gpu_workload(key)
     # ---- headline: W untimed steps, exactly K timed steps -----------------
     launches = built.launches(m.sets[0])
@@ -205,10 +212,10 @@ def main():
 
     line = {
         "metric": "best-config TFLOPS + % of MI355X roofline per op vs CPU llvm baseline",
-        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": value, "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name + " (BASELINE.json configs[1])", "task_key": key,
+        "config": {"workload": name + (" (BASELINE.json configs[1])" if headline == HEADLINE else ""), "task_key": key,
                    "tuned_config": json.loads(json.dumps(plan.configs)),
                    "device": props["name"], "arch": props["arch"]},
         "roofline": roof, "cpu_baseline": cpu, "per_config": per_config,

@@ -8,9 +8,13 @@ reference calls into TVM's runtime: ``tvm.build`` / ``export_library`` /
 There is no CPU fallback: if the shared library cannot be loaded, or a device
 call fails, an exception is raised.
 """
+import atexit
 import ctypes
 import hashlib
+import json
 import os
+import subprocess
+import sys
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -154,11 +158,53 @@ def code_key(src, opts, arch=DEFAULT_ARCH):
     return h.hexdigest()[:32]
 
 
-def compile_to_code(src, opts=(), arch=DEFAULT_ARCH, use_cache=True):
+_worker = None
+_worker_lock = threading.Lock()
+
+
+def _stop_worker():
+    global _worker
+    if _worker is not None:
+        try:
+            _worker.stdin.close()
+            _worker.wait(timeout=5)
+        except Exception:  # noqa: BLE001
+            _worker.kill()
+        _worker = None
+
+
+def _compile_out_of_process(src, opts, arch):
+    """Compile through the compile server (see compile_worker.py)."""
+    global _worker
+    with _worker_lock:
+        if _worker is None or _worker.poll() is not None:
+            env = dict(os.environ)
+            env["PYTHONPATH"] = os.path.dirname(_HERE) + os.pathsep + env.get("PYTHONPATH", "")
+            env["FLEXTENSOR_AMD_KCACHE"] = CACHE_DIR
+            _worker = subprocess.Popen([sys.executable, "-m", "flextensor_amd.compile_worker"],
+                                       stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                                       universal_newlines=True, env=env)
+            atexit.register(_stop_worker)
+        _worker.stdin.write(json.dumps({"src": src, "opts": list(opts), "arch": arch,
+                                        "cache_dir": CACHE_DIR}) + "\n")
+        _worker.stdin.flush()
+        line = _worker.stdout.readline()
+    if not line:
+        raise RuntimeError_("compile server died")
+    rep = json.loads(line)
+    if not rep.get("ok"):
+        raise RuntimeError_("ftr_compile_to_code: %s" % rep.get("error"))
+    with open(rep["path"], "rb") as f:
+        return f.read()
+
+
+def compile_to_code(src, opts=(), arch=DEFAULT_ARCH, use_cache=True, _in_process=False):
     """HIP source -> code object bytes (hiprtc, no device needed).
 
     Results are cached on disk under CACHE_DIR, keyed by a hash of the source,
-    the options and the architecture.
+    the options and the architecture. When PyTorch is loaded in this process
+    the compile runs in the compile server process instead (compile_worker.py)
+    so that the ROCm installation's compiler is used, not PyTorch's copy.
     """
     opts = list(opts)
     path = None
@@ -169,6 +215,8 @@ def compile_to_code(src, opts=(), arch=DEFAULT_ARCH, use_cache=True):
                 data = f.read()
             if data:
                 return data
+    if "torch" in sys.modules and not _in_process:
+        return _compile_out_of_process(src, opts, arch)
     code = ctypes.c_void_p()
     size = ctypes.c_size_t()
     rc = lib().ftr_compile_to_code(src.encode(), arch.encode(), _opt_array(opts),

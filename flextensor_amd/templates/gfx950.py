@@ -146,7 +146,7 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     space.add_subspace("xcd_remap", EnumSpace([[0], [1]]), "reorder")
     return space
@@ -179,16 +179,23 @@ def generate_space(op):
 # --------------------------------------------------------------------------
 
 SPECIAL_DEFAULTS = {
-    "lds_pad": [4, 8],     # fp32: [APAD, BPAD] floats; int8: [PAD bytes / 4, -]
+    # fp32: [APAD, BPAD] in floats; APAD -1 = unpadded, XOR-swizzled A tile;
+    # BPAD -1 = the padding that spreads the k-groups of one MFMA operand read
+    # over disjoint banks (4 floats for 16x16x4, 8 for 32x32x2).
+    # int8: [PAD bytes / 4, unused]
+    "lds_pad": [4, -1],
     "nt_store": [0],
 }
+
+# unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles)
+PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3)}
 
 
 def special_knobs(kind):
     """Enumerated knobs a task of this operator kind carries by default; they
     are attached with Task.set_specific_space and searched at graph level."""
     if kind in ("gemm", "conv2d_nchw"):
-        return {"lds_pad": [[4, 8], [4, 4], [0, 0], [4, 16], [8, 8]]}
+        return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
         return {"lds_pad": [[4, 0], [8, 0], [0, 0]], "nt_store": [[0], [1]]}
     if kind == "depthwise_conv2d_nchw":
@@ -219,7 +226,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     rd = _one(config, "reduce", 1, op.kind)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
-    stages = int((config.get("unroll") or [[2, 1]])[0][0])
+    depth = int((config.get("unroll") or [[2, 1]])[0][0])
+    if depth not in PIPELINE or (view.dtype == "int8" and depth > 2):
+        raise InvalidConfig("pipeline depth %d is not available" % depth)
+    stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
     xcd = int((config.get("reorder") or [[1]])[0][0])
     i8 = view.dtype == "int8"
@@ -228,8 +238,6 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         raise InvalidConfig("MFMA edge must be 16 or 32 and equal on both axes")
     if min(wm, rm, wn, rn, splitk, kiters, bk, group_m) < 1:
         raise InvalidConfig("non-positive factor")
-    if stages not in (1, 2):
-        raise InvalidConfig("LDS stages must be 1 or 2")
     nwaves = wm * wn
     if nwaves * 64 > MAX_THREADS:
         raise InvalidConfig("more than 16 wavefronts per workgroup")
@@ -269,7 +277,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     if bk % kblk != 0:
         raise InvalidConfig("BK must be a multiple of %d for this MFMA shape" % kblk)
     apad, bpad = [int(x) for x in _special(special, "lds_pad")[:2]]
-    if apad % 4 != 0 or bpad % 4 != 0:
+    if bpad < 0:
+        bpad = 4 if mfm == 16 else 8
+    if apad < -1 or (apad >= 0 and apad % 4 != 0) or bpad % 4 != 0:
         raise InvalidConfig("fp32 LDS padding must keep 16-byte alignment")
     av = 4 if view.K % 4 == 0 else 1
     if view.mode == 0:
@@ -278,7 +288,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         bv = av
     else:
         bv = 1
-    sa = bk + apad
+    sa = bk + max(apad, 0)
     if view.mode == 2:
         lds_b = bn * sa
     else:
@@ -289,9 +299,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     # staging registers for the global->LDS copy must stay reasonable
     ea = ceil_div(bm * bk // av, nt)
     eb = ceil_div((bn * bk) // bv, nt)
-    if (ea * av + eb * bv) > 128:
+    if (ea * av + eb * bv) * pd > 160:
         raise InvalidConfig("global->LDS staging needs too many registers")
-    D.update(MODE=view.mode, SPLITK=splitk, APAD=apad, BPAD=bpad, AV=av, BV=bv)
+    D.update(MODE=view.mode, SPLITK=splitk, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
     specs = []
     if view.mode == 1:
         conv = dict(view.conv)

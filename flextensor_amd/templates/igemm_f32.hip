@@ -17,16 +17,22 @@
 //   WAVES_M/N       wavefronts per workgroup along M / N
 //   REP_M/N         MFMA tiles per wavefront along M / N
 //   BK              K extent of one LDS tile
-//   STAGES          1 or 2 LDS buffers (2 = global loads of tile t+1 overlap
-//                   the MFMAs of tile t)
+//   STAGES          1 or 2 LDS buffers (2 = the LDS stores of tile t+1 need no
+//                   extra barrier against the reads of tile t)
+//   PD              prefetch distance: global loads of tile t+PD are in
+//                   flight (in PD register sets) while tile t is multiplied
 //   SPLITK          grid-level split of K; partial sums meet with float
 //                   atomics in C, which the caller zero-fills first
 //   GROUP_M         tile-traversal group height (L2 locality)
 //   XCD_REMAP       1: consecutive logical tiles stay on one XCD
-//   APAD / BPAD     LDS row padding in floats
+//   APAD / BPAD     LDS row padding in floats; APAD = -1 selects an unpadded
+//                   A tile whose 16-byte chunks are XOR-swizzled by row
 //
 // LDS layout: As[BM][BK+APAD] (k contiguous, read as one 128-bit load per
 // lane per 4 k-steps), Bs[BK][BN+BPAD] (n contiguous, read as 32-bit loads).
+// With the swizzle, chunk c of row r lives at chunk c ^ swz(r): 16 lanes that
+// read (or write) the same logical chunk of 16 consecutive rows touch 16
+// different groups of four banks.
 // Within a k-block of 4*KL values, lane group g of an MFMA takes
 // k = 4*g + s at step s for both operands, so the sum over k is unchanged.
 
@@ -44,6 +50,7 @@
 #define REP_N FT_REP_N
 #define BK FT_BK
 #define STAGES FT_STAGES
+#define PD FT_PD
 #define SPLITK FT_SPLITK
 #define GROUP_M FT_GROUP_M
 #define XCD_REMAP FT_XCD_REMAP
@@ -76,9 +83,28 @@ typedef f32x4 acc_t;
 #define BM (WAVES_M * REP_M * MFMA)
 #define BN (WAVES_N * REP_N * MFMA)
 #define NT (WAVES_M * WAVES_N * 64)
+#if APAD < 0
+#define ASWZ 1
+#define SA (BK)
+#else
+#define ASWZ 0
 #define SA (BK + APAD)
+#endif
+/* chunk swizzle of a k-contiguous tile: CRW 16-byte chunks per row */
+#define CRW (BK / 4)
+#if ASWZ
+#if CRW >= 16
+#define SWZ(row) ((row) & 15)
+#else
+#define SWZ(row) (((row) / (16 / CRW)) & (CRW - 1))
+#endif
+#else
+#define SWZ(row) 0
+#endif
+/* element column c of `row` -> physical column */
+#define ACOL(row, c) (((((c) >> 2) ^ SWZ(row)) << 2) | ((c) & 3))
 #if MODE == 2
-#define SB (BK + APAD)            /* Bs[BN][SB], k contiguous like As */
+#define SB (SA)                   /* Bs[BN][SB], k contiguous like As */
 #define BS_FLOATS (BN * SB)
 #else
 #define SB (BN + BPAD)            /* Bs[BK][SB], n contiguous */
@@ -209,10 +235,10 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     }
 #endif
 
-    avec_t areg[EA];
-    bvec_t breg[EB];
+    avec_t areg[PD][EA];
+    bvec_t breg[PD][EB];
 
-    auto load_global = [&](int kt) {
+    auto load_global = [&](int kt, int set) {
         const int k0 = kbase + kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
@@ -221,8 +247,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
             if (M % BM != 0) ok = ok && (m < M);
             if (KP != K) ok = ok && (k < K);
-            if (ok) areg[e] = *reinterpret_cast<const avec_t*>(A + (size_t)m * K + k);
-            else areg[e] = (avec_t)(0.0f);
+            if (ok) areg[set][e] = *reinterpret_cast<const avec_t*>(A + (size_t)m * K + k);
+            else areg[set][e] = (avec_t)(0.0f);
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
@@ -232,16 +258,16 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
             if (N % BN != 0) ok = ok && (n < N);
             if (KP != K) ok = ok && (k < K);
-            if (ok) breg[e] = *reinterpret_cast<const bvec_t*>(B + (size_t)n * K + k);
-            else breg[e] = (bvec_t)(0.0f);
+            if (ok) breg[set][e] = *reinterpret_cast<const bvec_t*>(B + (size_t)n * K + k);
+            else breg[set][e] = (bvec_t)(0.0f);
 #elif MODE == 0
             const int k = k0 + b_row[e];
             const int n = n0 + b_col[e];
             bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
             if (N % BN != 0) ok = ok && (n < N);
             if (KP != K) ok = ok && (k < K);
-            if (ok) breg[e] = *reinterpret_cast<const bvec_t*>(B + (size_t)k * N + n);
-            else breg[e] = (bvec_t)(0.0f);
+            if (ok) breg[set][e] = *reinterpret_cast<const bvec_t*>(B + (size_t)k * N + n);
+            else breg[set][e] = (bvec_t)(0.0f);
 #else
             const int k = k0 + b_row[e];
             const int c = k / (CR * CS);
@@ -250,21 +276,25 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int iw = px_w[e] + (rs % CS) * CDIL;
             bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
             if (KP != K) ok = ok && (k < K);
-            breg[e] = ok ? B[px_off[e] + c * (CH * CW) + ih * CW + iw] : 0.0f;
+            breg[set][e] = ok ? B[px_off[e] + c * (CH * CW) + ih * CW + iw] : 0.0f;
 #endif
         }
     };
 
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](int buf, int set) {
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
             if ((A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS))
-                *reinterpret_cast<avec_t*>(&As[buf][a_row[e] * SA + a_col[e]]) = areg[e];
+                *reinterpret_cast<avec_t*>(&As[buf][a_row[e] * SA + ACOL(a_row[e], a_col[e])]) = areg[set][e];
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
             if ((B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS))
-                *reinterpret_cast<bvec_t*>(&Bs[buf][b_row[e] * SB + b_col[e]]) = breg[e];
+#if MODE == 2
+                *reinterpret_cast<bvec_t*>(&Bs[buf][b_row[e] * SB + ACOL(b_row[e], b_col[e])]) = breg[set][e];
+#else
+                *reinterpret_cast<bvec_t*>(&Bs[buf][b_row[e] * SB + b_col[e]]) = breg[set][e];
+#endif
         }
     };
 
@@ -276,9 +306,11 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             acc[i][j] = (acc_t)(0.0f);
 
     auto compute = [&](int buf) {
-        const float* as = &As[buf][(wm * REP_M * MFMA + li) * SA + 4 * lg];
+        const int arow = wm * REP_M * MFMA + li;   /* + i*MFMA: SWZ is the same when MFMA % 16 == 0 */
+        const float* as = &As[buf][arow * SA];
 #if MODE == 2
-        const float* bs = &Bs[buf][(wn * REP_N * MFMA + li) * SB + 4 * lg];
+        const int brow = wn * REP_N * MFMA + li;
+        const float* bs = &Bs[buf][brow * SB];
 #else
         const float* bs = &Bs[buf][(4 * lg) * SB + wn * REP_N * MFMA + li];
 #endif
@@ -287,12 +319,12 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             f32x4 a[REP_M];
 #pragma unroll
             for (int i = 0; i < REP_M; ++i)
-                a[i] = *reinterpret_cast<const f32x4*>(as + i * MFMA * SA + kb);
+                a[i] = *reinterpret_cast<const f32x4*>(as + i * MFMA * SA + ACOL(arow + i * MFMA, kb + 4 * lg));
 #if MODE == 2
             f32x4 b4[REP_N];
 #pragma unroll
             for (int j = 0; j < REP_N; ++j)
-                b4[j] = *reinterpret_cast<const f32x4*>(bs + j * MFMA * SB + kb);
+                b4[j] = *reinterpret_cast<const f32x4*>(bs + j * MFMA * SB + ACOL(brow + j * MFMA, kb + 4 * lg));
 #endif
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
@@ -314,28 +346,28 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     };
 
     /* ---- main loop ------------------------------------------------------ */
-    load_global(0);
-    store_lds(0);
+    /* Tile t travels global -> register set t % PD -> LDS buffer -> MFMA.
+     * While tile kt is multiplied, tiles kt+1 .. kt+PD are in registers or in
+     * flight; tile kt+1 is written to LDS right after the MFMAs of tile kt. */
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+        if (p < KT) load_global(p, p);
+    store_lds(0, 0);
     __syncthreads();
-#if STAGES == 2
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) load_global(kt + 1);
-        compute(cur);
-        if (kt + 1 < KT) store_lds(cur ^ 1);
-        __syncthreads();
-    }
-#else
-    for (int kt = 0; kt < KT; ++kt) {
-        if (kt + 1 < KT) load_global(kt + 1);
-        compute(0);
-        __syncthreads();
-        if (kt + 1 < KT) {
-            store_lds(0);
-            __syncthreads();
+    for (int kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+        for (int u = 0; u < PD; ++u) {
+            const int kt = kt0 + u;
+            if (kt < KT) {
+                const int cur = (STAGES == 2) ? (kt & 1) : 0;
+                if (kt + PD < KT) load_global(kt + PD, u);
+                compute(cur);
+                if (STAGES == 1) __syncthreads();
+                if (kt + 1 < KT) store_lds((STAGES == 2) ? (cur ^ 1) : 0, (u + 1) % PD);
+                __syncthreads();
+            }
         }
     }
-#endif
 
     /* ---- epilogue: accumulators -> C ----------------------------------- */
 #pragma unroll

@@ -105,7 +105,7 @@ def test_lowering_rejects_bad_configs():
         _gemm_cfg([2, 2, 8, 32], [2, 2, 8, 32], [1, 64, 16]),     # 1024 accumulators
         _gemm_cfg([8, 8, 1, 16], [8, 8, 1, 16], [1, 64, 16]),     # 64 wavefronts
         _gemm_cfg([32, 2, 1, 16], [32, 2, 1, 16], [1, 128, 8]),   # BK < 16 with 16x16x4
-        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=3),
+        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=5),
     ]
     for cfg in bad:
         with pytest.raises(gfx950.InvalidConfig):

@@ -234,36 +234,51 @@ class Scheduler(object):
         self.timeout = old_timeout
 
     def _seed(self, configs, type_keys):
-        """Measure the template's default config first (when it is a point of
-        the space) so that the walk has a sane starting point."""
+        """Measure known-good points first so that the walk starts from them:
+        the template's default config and, when the task has one, the entry of
+        the shipped tuned log (points that are not in the space are skipped)."""
         if self.op_pos is None:
             return
         ops, _ = self.task.func(*self.task.args)
         op = flatten_graph(ops)[0][self.op_pos]
+        candidates = []
         try:
-            cfg = gfx950.default_config(op)
+            candidates.append(gfx950.default_config(op))
         except Exception:  # noqa: BLE001
-            return
-        indices = {}
-        for type_key in type_keys:
-            names = self.space.types[type_key]
-            ents = cfg.get(type_key, [])
-            if len(names) != len(ents):
-                return
-            for name, ent in zip(names, ents):
-                try:
-                    indices[name] = self.space.subspaces[name].static_entities.index(list(ent))
-                except ValueError:
-                    return
-        if self.walker_group.ever_met(indices):
-            return
-        res = self.parallel_evaluate(configs, [self.walker_group.to_config(indices)],
-                                     number=self.number)
-        self._log("seed [%.6f] [ %.6f ]" % (time.time(), res[0]))
-        if res[0] < float("inf"):
-            self.walker_group.record(indices, res[0])
-        else:
-            self.walker_group.visit.add(str(indices))
+            pass
+        try:
+            from .tuned import lookup
+            shipped = lookup(self.task_key)
+            if shipped is not None and self.op_pos < len(shipped.op_config_lst):
+                candidates.append(shipped.op_config_lst[self.op_pos])
+        except Exception:  # noqa: BLE001
+            pass
+        for cfg in candidates:
+            indices = {}
+            ok = True
+            for type_key in type_keys:
+                names = self.space.types[type_key]
+                ents = cfg.get(type_key, []) if cfg else []
+                if len(names) != len(ents):
+                    ok = False
+                    break
+                for name, ent in zip(names, ents):
+                    try:
+                        indices[name] = self.space.subspaces[name].static_entities.index(list(ent))
+                    except ValueError:
+                        ok = False
+                        break
+                if not ok:
+                    break
+            if not ok or not indices or self.walker_group.ever_met(indices):
+                continue
+            res = self.parallel_evaluate(configs, [self.walker_group.to_config(indices)],
+                                         number=self.number)
+            self._log("seed [%.6f] [ %.6f ]" % (time.time(), res[0]))
+            if res[0] < float("inf"):
+                self.walker_group.record(indices, res[0])
+            else:
+                self.walker_group.visit.add(str(indices))
 
     def _random_schedule(self, configs, type_keys, use_model=False):
         for trial in range(self.trial):

@@ -12,9 +12,12 @@
 //   REP_M/N     MFMA tiles per wavefront along M / N
 //   BK          bytes of K per LDS tile (multiple of the MFMA K)
 //   STAGES      1 or 2 LDS buffers
+//   PD          prefetch distance: global loads of tile t+PD are in flight
+//               (in PD register sets) while tile t is multiplied
 //   GROUP_M     tile-traversal group height (L2 locality)
 //   XCD_REMAP   1: consecutive logical tiles stay on one XCD
-//   PAD         LDS row padding in bytes (multiple of 16)
+//   PAD         LDS row padding in bytes (multiple of 16); -1 selects
+//               unpadded rows whose 16-byte chunks are XOR-swizzled by row
 //   NT_STORE    1: non-temporal stores for C
 //
 // Both operands live in LDS as [rows][BK+PAD] bytes and are read as one
@@ -36,6 +39,7 @@
 #define REP_N FT_REP_N
 #define BK FT_BK
 #define STAGES FT_STAGES
+#define PD FT_PD
 #define GROUP_M FT_GROUP_M
 #define XCD_REMAP FT_XCD_REMAP
 #define PAD FT_PAD
@@ -61,7 +65,21 @@ typedef i32x4 acc_t;
 #define BM (WAVES_M * REP_M * MFMA)
 #define BN (WAVES_N * REP_N * MFMA)
 #define NT (WAVES_M * WAVES_N * 64)
-#define SROW (BK + PAD)           /* LDS row stride in bytes */
+#define CRW (BK / 16)             /* 16-byte chunks per LDS row */
+#if PAD < 0
+#define SROW (BK)                 /* LDS row stride in bytes */
+#if CRW >= 16
+#define SWZ(row) ((row) & 15)
+#else
+#define SWZ(row) (((row) / (16 / CRW)) & (CRW - 1))
+#endif
+#else
+#define SROW (BK + PAD)
+#define SWZ(row) 0
+#endif
+/* byte column c (multiple of 16) of `row` -> physical byte column */
+#define PCOL(row, c) (((((c) >> 4) ^ SWZ(row)) << 4))
+#define OOB 0x80000000u
 #define TILES_M ((M + BM - 1) / BM)
 #define TILES_N ((N + BN - 1) / BN)
 /* KP = K rounded up to a multiple of 64 (host checks KP % BK == 0 and
@@ -71,7 +89,7 @@ typedef i32x4 acc_t;
 #if BK % MFMA_K != 0
 #error "BK must be a multiple of the MFMA K extent"
 #endif
-#if PAD % 16 != 0
+#if PAD >= 0 && PAD % 16 != 0
 #error "PAD must be a multiple of 16 bytes"
 #endif
 
@@ -124,39 +142,55 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         b_col[e] = (q % CHUNKS_ROW) * 16;
     }
 
-    i32x4 areg[EA], breg[EB];
+    /* raw buffer loads: an element that must read as zero (edge tile, idle
+     * lane, K tail) gets an offset beyond the buffer and loads 0 */
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<signed char*>(A), 0, M * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<signed char*>(B), 0, N * K, 0x00020000);
+    unsigned a_voff[EA], b_voff[EB];
+#pragma unroll
+    for (int e = 0; e < EA; ++e) {
+        const int m = m0 + a_row[e];
+        bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
+        if (M % BM != 0) ok = ok && (m < M);
+        a_voff[e] = ok ? (unsigned)(m * K + a_col[e]) : OOB;
+    }
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+        const int n = n0 + b_row[e];
+        bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
+        if (N % BN != 0) ok = ok && (n < N);
+        b_voff[e] = ok ? (unsigned)(n * K + b_col[e]) : OOB;
+    }
 
-    auto load_global = [&](int kt) {
+    i32x4 areg[PD][EA], breg[PD][EB];
+
+    auto load_global = [&](int kt, int set) {
         const int k0 = kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
-            const int m = m0 + a_row[e];
-            bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
-            if (M % BM != 0) ok = ok && (m < M);
-            if (KP != K) ok = ok && (k0 + a_col[e] < K);
-            if (ok) areg[e] = *reinterpret_cast<const i32x4*>(A + (size_t)m * K + k0 + a_col[e]);
-            else areg[e] = (i32x4)(0);
+            unsigned vo = a_voff[e];
+            if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+            areg[set][e] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (int)vo, k0, 0));
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
-            const int n = n0 + b_row[e];
-            bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
-            if (N % BN != 0) ok = ok && (n < N);
-            if (KP != K) ok = ok && (k0 + b_col[e] < K);
-            if (ok) breg[e] = *reinterpret_cast<const i32x4*>(B + (size_t)n * K + k0 + b_col[e]);
-            else breg[e] = (i32x4)(0);
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
+            breg[set][e] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)vo, k0, 0));
         }
     };
 
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](int buf, int set) {
 #pragma unroll
         for (int e = 0; e < EA; ++e)
             if ((A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS))
-                *reinterpret_cast<i32x4*>(&As[buf][a_row[e] * SROW + a_col[e]]) = areg[e];
+                *reinterpret_cast<i32x4*>(&As[buf][a_row[e] * SROW + PCOL(a_row[e], a_col[e])]) = areg[set][e];
 #pragma unroll
         for (int e = 0; e < EB; ++e)
             if ((B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS))
-                *reinterpret_cast<i32x4*>(&Bs[buf][b_row[e] * SROW + b_col[e]]) = breg[e];
+                *reinterpret_cast<i32x4*>(&Bs[buf][b_row[e] * SROW + PCOL(b_row[e], b_col[e])]) = breg[set][e];
     };
 
     acc_t acc[REP_M][REP_N];
@@ -167,17 +201,19 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             acc[i][j] = (acc_t)(0);
 
     auto compute = [&](int buf) {
-        const signed char* as = &As[buf][(wm * REP_M * MFMA + li) * SROW + 16 * lg];
-        const signed char* bs = &Bs[buf][(wn * REP_N * MFMA + li) * SROW + 16 * lg];
+        const int arow = wm * REP_M * MFMA + li;
+        const int brow = wn * REP_N * MFMA + li;
+        const signed char* as = &As[buf][arow * SROW];
+        const signed char* bs = &Bs[buf][brow * SROW];
 #pragma unroll
         for (int kk = 0; kk < BK; kk += MFMA_K) {
             i32x4 a[REP_M], b[REP_N];
 #pragma unroll
             for (int i = 0; i < REP_M; ++i)
-                a[i] = *reinterpret_cast<const i32x4*>(as + i * MFMA * SROW + kk);
+                a[i] = *reinterpret_cast<const i32x4*>(as + i * MFMA * SROW + PCOL(arow + i * MFMA, kk + 16 * lg));
 #pragma unroll
             for (int j = 0; j < REP_N; ++j)
-                b[j] = *reinterpret_cast<const i32x4*>(bs + j * MFMA * SROW + kk);
+                b[j] = *reinterpret_cast<const i32x4*>(bs + j * MFMA * SROW + PCOL(brow + j * MFMA, kk + 16 * lg));
 #pragma unroll
             for (int i = 0; i < REP_M; ++i)
 #pragma unroll
@@ -186,28 +222,29 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         }
     };
 
-    load_global(0);
-    store_lds(0);
+    /* tile t: global -> register set t % PD -> LDS buffer -> MFMA */
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+        if (p < KT) load_global(p, p);
+    store_lds(0, 0);
     __syncthreads();
-#if STAGES == 2
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) load_global(kt + 1);
-        compute(cur);
-        if (kt + 1 < KT) store_lds(cur ^ 1);
-        __syncthreads();
-    }
-#else
-    for (int kt = 0; kt < KT; ++kt) {
-        if (kt + 1 < KT) load_global(kt + 1);
-        compute(0);
-        __syncthreads();
-        if (kt + 1 < KT) {
-            store_lds(0);
-            __syncthreads();
+    for (int kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+        for (int u = 0; u < PD; ++u) {
+            const int kt = kt0 + u;
+            if (kt < KT) {
+                const int cur = (STAGES == 2) ? (kt & 1) : 0;
+                if (kt + PD < KT) load_global(kt + PD, u);
+                /* keep the prefetch at the top of the iteration: without this
+                 * fence the scheduler sinks the loads down to their use */
+                __builtin_amdgcn_sched_barrier(0);
+                compute(cur);
+                if (STAGES == 1) __syncthreads();
+                if (kt + 1 < KT) store_lds((STAGES == 2) ? (cur ^ 1) : 0, (u + 1) % PD);
+                __syncthreads();
+            }
         }
     }
-#endif
 
 #pragma unroll
     for (int i = 0; i < REP_M; ++i) {

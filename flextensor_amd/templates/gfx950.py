@@ -126,7 +126,7 @@ class GemmView(object):
         self.KP = ceil_div(self.K, 64) * 64 if self.dtype == "int8" else ceil_div(self.K, 16) * 16
 
 
-F32_BK = (8, 16, 32, 64)
+F32_BK = (8, 16, 32, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
 I8_BK = (64, 128, 256)
 
 
@@ -146,9 +146,11 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
-    space.add_subspace("xcd_remap", EnumSpace([[0], [1]]), "reorder")
+    # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
+    space.add_subspace("xcd_remap", EnumSpace([[1, 0], [0, 0]] if i8 else [[1, 0], [0, 0], [1, 1], [0, 1]]),
+                       "reorder")
     return space
 
 
@@ -197,7 +199,7 @@ def special_knobs(kind):
     if kind in ("gemm", "conv2d_nchw"):
         return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
-        return {"lds_pad": [[4, 0], [8, 0], [0, 0]], "nt_store": [[0], [1]]}
+        return {"lds_pad": [[4, 0], [-1, 0], [8, 0]], "nt_store": [[0], [1]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1]]}
     return {}
@@ -227,18 +229,24 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE or (view.dtype == "int8" and depth > 2):
+    if depth not in PIPELINE:
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
-    xcd = int((config.get("reorder") or [[1]])[0][0])
+    ro = list((config.get("reorder") or [[1, 0]])[0]) + [0]
+    xcd, in_wg = int(ro[0]), int(ro[1])
     i8 = view.dtype == "int8"
+    waves_k = 1
+    if in_wg and splitk > 1:
+        if i8:
+            raise InvalidConfig("int8 GEMM does not split K")
+        waves_k, splitk = splitk, 1
 
     if mfm != mfn or mfm not in (16, 32):
         raise InvalidConfig("MFMA edge must be 16 or 32 and equal on both axes")
     if min(wm, rm, wn, rn, splitk, kiters, bk, group_m) < 1:
         raise InvalidConfig("non-positive factor")
-    nwaves = wm * wn
+    nwaves = wm * wn * waves_k
     if nwaves * 64 > MAX_THREADS:
         raise InvalidConfig("more than 16 wavefronts per workgroup")
     bm, bn = wm * rm * mfm, wn * rn * mfn
@@ -247,9 +255,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     nacc = rm * rn * (mfm * mfm // 64)
     if nacc > MAX_ACC_REGS:
         raise InvalidConfig("accumulators need %d registers per lane" % nacc)
-    if splitk * kiters * bk != view.KP:
+    if splitk * waves_k * kiters * bk != view.KP:
         raise InvalidConfig("reduce split does not multiply to K")
-    nt = nwaves * 64
+    nt = wm * wn * 64          # threads of one k-group
     D = dict(M=view.M, N=view.N, K=view.K, KP=view.KP, MFMA=mfm, WAVES_M=wm, WAVES_N=wn, REP_M=rm,
              REP_N=rn, BK=bk, STAGES=stages, GROUP_M=group_m, XCD_REMAP=xcd)
 
@@ -261,13 +269,18 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
             raise InvalidConfig("BK must be a multiple of the MFMA K extent")
         if view.K % 16 != 0:
             raise InvalidConfig("int8 GEMM needs K to be a multiple of 16")
-        pad = int(_special(special, "lds_pad")[0]) * 4
-        if pad % 16 != 0:
+        pad = int(_special(special, "lds_pad")[0])
+        pad = -1 if pad < 0 else pad * 4
+        if pad >= 0 and pad % 16 != 0:
             raise InvalidConfig("int8 LDS padding must be a multiple of 16 bytes")
-        lds = stages * (bm + bn) * (bk + pad)
+        if view.M * view.K >= 2 ** 31 or view.N * view.K >= 2 ** 31:
+            raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
+        if (ceil_div(bm * bk // 16, nt) + ceil_div(bn * bk // 16, nt)) * 4 * pd > 160:
+            raise InvalidConfig("global->LDS staging needs too many registers")
+        lds = stages * (bm + bn) * (bk + max(pad, 0))
         if lds > LDS_BYTES:
             raise InvalidConfig("LDS tile needs %d bytes" % lds)
-        D.update(PAD=pad, NT_STORE=int(_special(special, "nt_store")[0]))
+        D.update(PAD=pad, PD=pd, NT_STORE=int(_special(special, "nt_store")[0]))
         grid = (gm * gn, 1, 1)
         spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])
@@ -288,12 +301,14 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         bv = av
     else:
         bv = 1
+    if apad < 0 and (bk & (bk - 1)) != 0:
+        apad = 4              # the chunk swizzle needs a power-of-two row
     sa = bk + max(apad, 0)
     if view.mode == 2:
         lds_b = bn * sa
     else:
         lds_b = bk * (bn + bpad)
-    lds = stages * 4 * (bm * sa + lds_b)
+    lds = max(waves_k * stages * 4 * (bm * sa + lds_b), (waves_k - 1) * nt * nacc * 4)
     if lds > LDS_BYTES:
         raise InvalidConfig("LDS tile needs %d bytes" % lds)
     # staging registers for the global->LDS copy must stay reasonable
@@ -301,7 +316,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     eb = ceil_div((bn * bk) // bv, nt)
     if (ea * av + eb * bv) * pd > 160:
         raise InvalidConfig("global->LDS staging needs too many registers")
-    D.update(MODE=view.mode, SPLITK=splitk, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
+    if max(view.M * view.K, view.K * view.N, view.M * view.N) * 4 >= 2 ** 31:
+        raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
+    D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
     specs = []
     if view.mode == 1:
         conv = dict(view.conv)
@@ -320,7 +337,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
                                 (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
                                 [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
     grid = (gm * gn * splitk, 1, 1)
-    specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt, 1, 1),
+    specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt * waves_k, 1, 1),
                             [("buf", a_name), ("buf", b_name), ("buf", out_name)]))
     return specs
 
@@ -402,32 +419,30 @@ def default_config(op):
         view = GemmView(op)
         i8 = view.dtype == "int8"
 
-        def tile(extent, want):
-            mf = 32 if extent >= 32 else 16
-            t = mf
+        def tile(extent, want, mf):
+            """[grid, waves, reps, mfma] with a tile close to ``want``."""
             w, r = 1, 1
             while w * r * mf * 2 <= want and w * r * mf * 2 <= max(extent, mf):
                 if w < 2:
                     w *= 2
                 else:
                     r *= 2
-            del t
             return [ceil_div(extent, w * r * mf), w, r, mf]
 
+        mf = 32 if min(view.M, view.N) >= 64 else 16
+        # the largest square-ish tile that still yields one workgroup per CU
         want = 256 if i8 else 128
-        tm, tn = tile(view.M, want), tile(view.N, want)
-        mf = min(tm[3], tn[3])
-        for t, ext in ((tm, view.M), (tn, view.N)):
-            if t[3] != mf:
-                t[2] *= t[3] // mf
-                t[3] = mf
-            t[0] = ceil_div(ext, t[1] * t[2] * t[3])
+        while True:
+            tm, tn = tile(view.M, want, mf), tile(view.N, want, mf)
+            if tm[0] * tn[0] >= 256 or want <= mf:
+                break
+            want //= 2
         cfg["spatial"] = [tm, tn]
         bks = I8_BK if i8 else F32_BK
         kblk = (32 if mf == 32 else 64) if i8 else 4 * (64 // mf)
         bk = None
         for cand in sorted(bks, reverse=True):
-            if view.KP % cand == 0 and cand % kblk == 0 and cand <= (64 if i8 else 16):
+            if view.KP % cand == 0 and cand % kblk == 0 and cand <= (64 if i8 else 32):
                 bk = cand
                 break
         if bk is None:
@@ -438,9 +453,9 @@ def default_config(op):
         if bk is None:
             raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
         cfg["reduce"] = [[1, view.KP // bk, bk]]
-        cfg["unroll"] = [[2, 1]]
+        cfg["unroll"] = [[2, 1]] if i8 else [[3, 1]]
         cfg["fuse"] = [[4]]
-        cfg["reorder"] = [[1]]
+        cfg["reorder"] = [[1, 0]]
     elif op.kind == "depthwise_conv2d_nchw":
         b, c, p, q = [x.extent for x in op.axis]
         th = 4 if p >= 4 else 1

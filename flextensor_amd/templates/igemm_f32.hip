@@ -23,6 +23,10 @@
 //                   flight (in PD register sets) while tile t is multiplied
 //   SPLITK          grid-level split of K; partial sums meet with float
 //                   atomics in C, which the caller zero-fills first
+//   WAVES_K         split of K inside the workgroup: WAVES_K groups of
+//                   WAVES_M*WAVES_N wavefronts each multiply their own K slice
+//                   through their own LDS tiles; the partial tiles are summed
+//                   through LDS at the end (no atomics, no zero fill)
 //   GROUP_M         tile-traversal group height (L2 locality)
 //   XCD_REMAP       1: consecutive logical tiles stay on one XCD
 //   APAD / BPAD     LDS row padding in floats; APAD = -1 selects an unpadded
@@ -52,6 +56,7 @@
 #define STAGES FT_STAGES
 #define PD FT_PD
 #define SPLITK FT_SPLITK
+#define WAVES_K FT_WAVES_K
 #define GROUP_M FT_GROUP_M
 #define XCD_REMAP FT_XCD_REMAP
 #define APAD FT_APAD
@@ -82,7 +87,8 @@ typedef f32x4 acc_t;
 #define KBLK (4 * KL)             /* k values per 128-bit A fragment round  */
 #define BM (WAVES_M * REP_M * MFMA)
 #define BN (WAVES_N * REP_N * MFMA)
-#define NT (WAVES_M * WAVES_N * 64)
+#define NT (WAVES_M * WAVES_N * 64)   /* threads of one k-group */
+#define NTW (NT * WAVES_K)             /* threads of the workgroup */
 #if APAD < 0
 #define ASWZ 1
 #define SA (BK)
@@ -115,7 +121,8 @@ typedef f32x4 acc_t;
 /* KP = K rounded up to a multiple of 16; the host checks KP % (SPLITK*BK) == 0.
  * When KP != K the tail is zero-filled by the load predicates. */
 #define KSPLIT_LEN (KP / SPLITK)
-#define KT (KSPLIT_LEN / BK)
+#define KGROUP_LEN (KSPLIT_LEN / WAVES_K)
+#define KT (KGROUP_LEN / BK)
 
 #if BK % KBLK != 0
 #error "BK must be a multiple of 4*(64/MFMA)"
@@ -150,6 +157,27 @@ typedef float bvec_t;
 #error "BV must be 1 or 4"
 #endif
 
+/* byte sizes of the operands (the host checks that each is below 2 GiB) */
+#define OOB 0x80000000u
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+static __device__ __forceinline__ float ld_f32(__amdgpu_buffer_rsrc_t r, unsigned vo, int so) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)vo, so, 0));
+}
+static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsigned vo, int so) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)vo, so, 0));
+}
+#if AV == 4
+#define LOAD_A ld_f32x4
+#else
+#define LOAD_A ld_f32
+#endif
+#if BV == 4
+#define LOAD_B ld_f32x4
+#else
+#define LOAD_B ld_f32
+#endif
+#define A_BYTES (M * K * 4)
+
 #if MODE == 1
 #define CB FT_CB
 #define CC FT_CC
@@ -165,19 +193,46 @@ typedef float bvec_t;
 /* conv geometry, all compile-time: input [CB][CC][CH][CW], kernel CR x CS,
  * stride CSTR, padding CPAD, dilation CDIL, output CP x CQ. */
 #define OHW (CP * CQ)
+#define B_BYTES (CB * CC * CH * CW * 4)
+/* When an LDS tile spans whole kernel windows (BK % (CR*CS) == 0) every
+ * gathered element keeps its tap (r, s) and its channel offset inside the
+ * tile for the whole K loop: the index arithmetic and the padding predicate
+ * are computed once and the loop only advances by a constant stride. */
+#if BK % (CR * CS) == 0
+#define KHOIST 1
+#else
+#define KHOIST 0
+#endif
 #if BV != 1
 #error "conv mode gathers scalars: BV must be 1"
 #endif
+#else
+#define B_BYTES (K * N * 4)
 #endif
 
-extern "C" __global__ __launch_bounds__(NT)
+#define A_FLOATS (BM * SA)
+#define TILE_FLOATS (WAVES_K * STAGES * (A_FLOATS + BS_FLOATS))
+#define RED_FLOATS ((WAVES_K - 1) * NT * REP_M * REP_N * NACC)
+#define SMEM_FLOATS (TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS)
+
+extern "C" __global__ __launch_bounds__(NTW)
 void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                float* __restrict__ C)
 {
-    __shared__ __attribute__((aligned(16))) float As[STAGES][BM * SA];
-    __shared__ __attribute__((aligned(16))) float Bs[STAGES][BS_FLOATS];
-
+    __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+    /* k-group of this wavefront (NT is a multiple of 64, so it is uniform
+     * over a wavefront; readfirstlane tells the compiler so) */
+#if WAVES_K > 1
+    const int kg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / NT));
+    const int tid = threadIdx.x - kg * NT;      /* thread index inside the k-group */
+#else
+    const int kg = 0;
     const int tid = threadIdx.x;
+#endif
+    float (*As)[A_FLOATS] = reinterpret_cast<float (*)[A_FLOATS]>(smem + kg * STAGES * A_FLOATS);
+    float (*Bs)[BS_FLOATS] = reinterpret_cast<float (*)[BS_FLOATS]>(
+        smem + WAVES_K * STAGES * A_FLOATS + kg * STAGES * BS_FLOATS);
+
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave / WAVES_N;
@@ -201,7 +256,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const int tile_n = rr / gsz;
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
-    const int kbase = kz * KSPLIT_LEN;
+    const int kbase = kz * KSPLIT_LEN + kg * KGROUP_LEN;
 
     /* ---- per-thread load coordinates ----------------------------------- */
     int a_row[EA], a_col[EA];
@@ -235,6 +290,47 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     }
 #endif
 
+    /* ---- global loads: raw buffer loads with hardware bounds checking --- */
+    /* Every element gets a byte offset computed once; an element that must
+     * read as zero (tile edge, zero padding, idle lane) gets an offset beyond
+     * the buffer, for which the load returns 0 without a branch. The part of
+     * the address that advances with the K loop is wave-uniform and goes into
+     * the scalar offset operand. */
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, A_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, B_BYTES, 0x00020000);
+    unsigned a_voff[EA], b_voff[EB];
+#pragma unroll
+    for (int e = 0; e < EA; ++e) {
+        const int m = m0 + a_row[e];
+        bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
+        if (M % BM != 0) ok = ok && (m < M);
+        a_voff[e] = ok ? (unsigned)(m * K + a_col[e]) * 4u : OOB;
+    }
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+        bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
+#if MODE == 2
+        const int n = n0 + b_row[e];
+        if (N % BN != 0) ok = ok && (n < N);
+        b_voff[e] = ok ? (unsigned)(n * K + b_col[e]) * 4u : OOB;
+#elif MODE == 0
+        const int n = n0 + b_col[e];
+        if (N % BN != 0) ok = ok && (n < N);
+        b_voff[e] = ok ? (unsigned)(b_row[e] * N + n) * 4u : OOB;
+#elif KHOIST
+        const int cl = b_row[e] / (CR * CS);
+        const int rs = b_row[e] % (CR * CS);
+        const int ih = px_h[e] + (rs / CS) * CDIL;
+        const int iw = px_w[e] + (rs % CS) * CDIL;
+        ok = ok && px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+        b_voff[e] = ok ? (unsigned)(px_off[e] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
+#else
+        b_voff[e] = OOB;  /* recomputed for every tile */
+#endif
+    }
+
     avec_t areg[PD][EA];
     bvec_t breg[PD][EB];
 
@@ -242,32 +338,24 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         const int k0 = kbase + kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
-            const int m = m0 + a_row[e];
-            const int k = k0 + a_col[e];
-            bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
-            if (M % BM != 0) ok = ok && (m < M);
-            if (KP != K) ok = ok && (k < K);
-            if (ok) areg[set][e] = *reinterpret_cast<const avec_t*>(A + (size_t)m * K + k);
-            else areg[set][e] = (avec_t)(0.0f);
+            unsigned vo = a_voff[e];
+            if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+            areg[set][e] = LOAD_A(rsrc_a, vo, k0 * 4);
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
 #if MODE == 2
-            const int n = n0 + b_row[e];
-            const int k = k0 + b_col[e];
-            bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
-            if (N % BN != 0) ok = ok && (n < N);
-            if (KP != K) ok = ok && (k < K);
-            if (ok) breg[set][e] = *reinterpret_cast<const bvec_t*>(B + (size_t)n * K + k);
-            else breg[set][e] = (bvec_t)(0.0f);
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
+            breg[set][e] = LOAD_B(rsrc_b, vo, k0 * 4);
 #elif MODE == 0
-            const int k = k0 + b_row[e];
-            const int n = n0 + b_col[e];
-            bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
-            if (N % BN != 0) ok = ok && (n < N);
-            if (KP != K) ok = ok && (k < K);
-            if (ok) breg[set][e] = *reinterpret_cast<const bvec_t*>(B + (size_t)k * N + n);
-            else breg[set][e] = (bvec_t)(0.0f);
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            breg[set][e] = LOAD_B(rsrc_b, vo, k0 * (N * 4));
+#elif KHOIST
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            breg[set][e] = LOAD_B(rsrc_b, vo, (k0 / (CR * CS)) * (CH * CW * 4));
 #else
             const int k = k0 + b_row[e];
             const int c = k / (CR * CS);
@@ -276,7 +364,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int iw = px_w[e] + (rs % CS) * CDIL;
             bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
             if (KP != K) ok = ok && (k < K);
-            breg[set][e] = ok ? B[px_off[e] + c * (CH * CW) + ih * CW + iw] : 0.0f;
+            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
+            breg[set][e] = LOAD_B(rsrc_b, vo, 0);
 #endif
         }
     };
@@ -361,6 +450,9 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             if (kt < KT) {
                 const int cur = (STAGES == 2) ? (kt & 1) : 0;
                 if (kt + PD < KT) load_global(kt + PD, u);
+                /* keep the prefetch at the top of the iteration: without this
+                 * fence the scheduler sinks the loads down to their use */
+                __builtin_amdgcn_sched_barrier(0);
                 compute(cur);
                 if (STAGES == 1) __syncthreads();
                 if (kt + 1 < KT) store_lds((STAGES == 2) ? (cur ^ 1) : 0, (u + 1) % PD);
@@ -368,6 +460,34 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             }
         }
     }
+
+#if WAVES_K > 1
+    /* ---- sum the k-groups' partial tiles through LDS --------------------- */
+    /* the last barrier of the main loop has passed: tile memory is free */
+    if (kg > 0) {
+        float* red = smem + (kg - 1) * (NT * REP_M * REP_N * NACC);
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v)
+                    red[((i * REP_N + j) * NACC + v) * NT + tid] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (kg > 0) return;
+#pragma unroll
+    for (int g = 1; g < WAVES_K; ++g) {
+        const float* red = smem + (g - 1) * (NT * REP_M * REP_N * NACC);
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v)
+                    acc[i][j][v] += red[((i * REP_N + j) * NACC + v) * NT + tid];
+    }
+#endif
 
     /* ---- epilogue: accumulators -> C ----------------------------------- */
 #pragma unroll

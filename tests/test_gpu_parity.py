@@ -41,11 +41,12 @@ def key_of(category, name, args):
     return Task(category, name, None, args, "rocm", 0).key
 
 
-def gcfg(M, N, K, wm, rm, wn, rn, mf, bk, sk=1, st=2, gm=4, xcd=1):
+def gcfg(M, N, K, wm, rm, wn, rn, mf, bk, sk=1, st=2, gm=4, xcd=1, wk=0):
+    """st = pipeline depth; wk=1: the sk K-partitions are wavefront groups of one workgroup."""
     c = {k: [] for k in KEYS}
     c["spatial"] = [[ceil_div(M, wm * rm * mf), wm, rm, mf], [ceil_div(N, wn * rn * mf), wn, rn, mf]]
     c["reduce"] = [[sk, K // (sk * bk), bk]]
-    c["unroll"], c["fuse"], c["reorder"] = [[st, 1]], [[gm]], [[xcd]]
+    c["unroll"], c["fuse"], c["reorder"] = [[st, 1]], [[gm]], [[xcd, wk]]
     return c
 
 
@@ -174,6 +175,12 @@ GEMM_CASES = [
     (200, 136, 328, dict(wm=2, rm=1, wn=1, rn=3, mf=32, bk=8)),      # ragged M, N; N % 4 == 0
     (96, 80, 67, dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=16)),        # N % 4 != 0 -> scalar loads
     (512, 1024, 128, dict(wm=4, rm=1, wn=1, rn=2, mf=32, bk=32, sk=8, gm=2)),
+    (256, 256, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=3)),                 # prefetch 2 tiles
+    (256, 512, 256, dict(wm=2, rm=2, wn=2, rn=1, mf=16, bk=16, st=4)),                 # prefetch 3 tiles
+    (200, 96, 328, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=16, st=4)),                  # KT < prefetch + ragged
+    (256, 512, 256, dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32, sk=4, wk=1, st=3)),     # in-workgroup split-K
+    (96, 256, 67, dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=16, sk=8, wk=1)),             # 8 k-groups, ragged
+    (128, 1024, 128, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=32, sk=2, wk=1, st=4)),    # big reduce buffer
 ]
 
 
@@ -229,6 +236,8 @@ CONV_CASES = [
     ((3, 6, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32)),   # dilation 2
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=32)),    # 1x1, N=392
     ((1, 3, 32, 32, 16, 7, 2, 3, 1, 1), dict(wm=1, rm=1, wn=4, rn=1, mf=16, bk=16)),   # 7x7 s2 p3, K=147
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=16, bk=16, sk=3, wk=1, st=3)),
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=32, sk=2, wk=1, st=4)),
 ]
 
 

@@ -70,8 +70,14 @@ def gpu_workload(key, seed=0):
     return built, m, s
 
 
-def kernel_ms(built, m, iters=200, warmup=20):
-    """Mean duration of one plan run, HIP events on the launch stream."""
+TIMED_WINDOW_MS = 2.5   # every workload is timed over about this much device time
+
+
+def kernel_ms(built, m, iters=None, warmup=20):
+    """Mean duration of one plan run, HIP events on the launch stream. The
+    number of timed launches is chosen so that every workload is measured
+    over the same wall window (a 6 us kernel and a 70 us kernel then see the
+    same clock/power conditions)."""
     import torch
     first = m.sets[0]
     built(*first)
@@ -79,6 +85,9 @@ def kernel_ms(built, m, iters=200, warmup=20):
     ok, metric = m.check(first[-1])
     if not ok:
         raise RuntimeError("tuned plan fails the correctness gate (metric %g)" % metric)
+    if iters is None:
+        probe = built.time(m.sets, warmup=warmup, iters=10)
+        iters = int(min(max(TIMED_WINDOW_MS / max(probe, 1e-4), 20), 1000))
     return built.time(m.sets, warmup=warmup, iters=iters), metric
 
 
@@ -156,7 +165,7 @@ def main():
     headline = HEADLINE if args.workload is None else [w[0] for w in WORKLOADS].index(args.workload)
     name, key, ops, nbytes, bound, dtype = WORKLOADS[headline]
     if dtype == "i8":
-        args.steps = min(args.steps, 500)
+        args.steps = min(args.steps, 100)
     built, m, plan = gpu_workload(key)
     # ---- headline: W untimed steps, exactly K timed steps -----------------
     launches = built.launches(m.sets[0])
@@ -175,7 +184,7 @@ def main():
     ok, metric = m.check(m.sets[0][-1])
     if not ok:
         raise RuntimeError("headline plan fails the correctness gate (metric %g)" % metric)
-    k_ms, _ = kernel_ms(built, m, iters=max(args.steps // 4, 50))
+    k_ms, _ = kernel_ms(built, m)
     roof = roofline(bound, dtype, ops, nbytes, k_ms)
     roof["kernel"] = plan.specs[-1].kernel
     roof["kernel_ms"] = k_ms
@@ -185,7 +194,7 @@ def main():
     if not args.only_headline:
         for (wname, wkey, wops, wbytes, wbound, wdtype) in WORKLOADS:
             b, mm, pl = gpu_workload(wkey)
-            ms, met = kernel_ms(b, mm, iters=100 if wdtype == "i8" else 300)
+            ms, met = kernel_ms(b, mm)
             r = roofline(wbound, wdtype, wops, wbytes, ms)
             entry = {"workload": wname, "ms": ms, "dtype": wdtype,
                      "throughput": wops / (ms * 1e-3) / 1e12,

@@ -11,7 +11,11 @@
 // H, then planes, so global reads and writes of a wavefront are contiguous.
 //
 // Knobs (-D constants): NT threads per workgroup, TH x TW outputs per lane,
-// NT_STORE (1: non-temporal stores for the output).
+// NT_STORE (1: non-temporal stores for the output), SHFL (1: the one-column
+// halo left and right of a lane's four columns comes from the neighbouring
+// lanes through DPP wavefront shifts instead of two more global loads; each
+// wavefront then uses a multiple of TILES_W lanes so that neighbours along W
+// are always in the same wavefront).
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
 // STR, PAD, DIL, FACT, CP x CQ output.
 
@@ -21,6 +25,7 @@
 #define TH FT_TH
 #define TW FT_TW
 #define NT_STORE FT_NT_STORE
+#define SHFL FT_SHFL
 #define CB FT_CB
 #define CC FT_CC
 #define CH FT_CH
@@ -55,21 +60,37 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #else
 #define VEC_OUT 0
 #endif
+#if SHFL
+#if !(VEC_IN && CS == 3 && DIL == 1 && PAD == 1 && TILES_W <= 64)
+#error "SHFL needs the 128-bit input path with a 3-wide kernel, dilation 1, padding 1"
+#endif
+#define LPW ((64 / TILES_W) * TILES_W)   /* lanes of a wavefront that carry work */
+#else
+#define LPW 64
+#endif
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                    float* __restrict__ O)
 {
+#if SHFL
+    const int lane = threadIdx.x & 63;
+    const int gid = ((blockIdx.x * NT + threadIdx.x) >> 6) * LPW + lane;
+    /* idle lanes stay alive (DPP reads their registers) but load and store nothing */
+    const bool live = (lane < LPW) && (gid < ITEMS);
+#else
     const int gid = blockIdx.x * NT + threadIdx.x;
     if (gid >= ITEMS) return;
+    const bool live = true;
+#endif
     const int tw = gid % TILES_W;
     const int th = (gid / TILES_W) % TILES_H;
     const int plane = gid / (TILES_W * TILES_H);
     const int b = plane / (CC * FACT);
     const int co = plane % (CC * FACT);
     const int ci = co / FACT;
-    const float* x = X + (size_t)(b * CC + ci) * (CH * CW);
-    const float* wp = Wt + (size_t)co * (CR * CS);
+    const float* x = X + (size_t)(live ? (b * CC + ci) : 0) * (CH * CW);
+    const float* wp = Wt + (size_t)(live ? co : 0) * (CR * CS);
     float* o = O + (size_t)plane * (CP * CQ);
 
     float wreg[CR][CS];
@@ -94,10 +115,23 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #pragma unroll
     for (int y = 0; y < IH_T; ++y) {
         const int ih = ih0 + y;
-        const bool row_ok = (unsigned)ih < (unsigned)CH;
+        const bool row_ok = live && (unsigned)ih < (unsigned)CH;
         const float* xr = x + ih * CW;
         float in[IW_T];
-#if VEC_IN
+#if SHFL
+        {
+            f32x4 v = (f32x4)(0.0f);
+            if (row_ok) v = *reinterpret_cast<const f32x4*>(xr + ow0);
+            /* column ow0-1 is the last column of the lane below, column ow0+4
+             * the first column of the lane above; image borders read zero */
+            const float v0 = v[0], v3 = v[3];
+            const int lft = __builtin_amdgcn_update_dpp(0, __float_as_int(v3), 0x138, 0xf, 0xf, false);
+            const int rgt = __builtin_amdgcn_update_dpp(0, __float_as_int(v0), 0x130, 0xf, 0xf, false);
+            in[0] = (tw > 0) ? __int_as_float(lft) : 0.0f;
+            in[1] = v[0]; in[2] = v[1]; in[3] = v[2]; in[4] = v[3];
+            in[5] = (tw < TILES_W - 1) ? __int_as_float(rgt) : 0.0f;
+        }
+#elif VEC_IN
         {
             f32x4 v = (f32x4)(0.0f);
             if (row_ok) v = *reinterpret_cast<const f32x4*>(xr + ow0);
@@ -134,6 +168,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         }
     }
 
+    if (!live) return;
 #pragma unroll
     for (int i = 0; i < TH; ++i) {
         const int oh = oh0 + i;

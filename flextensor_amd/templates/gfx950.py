@@ -187,6 +187,7 @@ SPECIAL_DEFAULTS = {
     # int8: [PAD bytes / 4, unused]
     "lds_pad": [4, -1],
     "nt_store": [0],
+    "halo_shfl": [0],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles)
@@ -199,9 +200,9 @@ def special_knobs(kind):
     if kind in ("gemm", "conv2d_nchw"):
         return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
-        return {"lds_pad": [[4, 0], [-1, 0], [8, 0]], "nt_store": [[0], [1]]}
+        return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1]]}
     if kind == "depthwise_conv2d_nchw":
-        return {"nt_store": [[0], [1]]}
+        return {"nt_store": [[0], [1]], "halo_shfl": [[0], [1]]}
     return {}
 
 
@@ -371,11 +372,21 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         raise InvalidConfig("lane patch needs too many registers")
     nt = waves * 64
     items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
-    D = dict(NT=nt, TH=th, TW=tw, NT_STORE=int(_special(special, "nt_store")[0]),
+    shfl = int(_special(special, "halo_shfl")[0])
+    tiles_w = ceil_div(q, tw)
+    if shfl:
+        vec_in = (tw == 4 and a["stride"][0] == 1 and w % 4 == 0 and q == w and pad + 4 <= iw_t)
+        if not (vec_in and s_ext == 3 and a["dilation"][0] == 1 and pad == 1 and tiles_w <= 64):
+            raise InvalidConfig("the shuffled halo needs the 128-bit input path of a 3x3 pad-1 layer")
+        lanes = (64 // tiles_w) * tiles_w
+        grid_x = ceil_div(ceil_div(items, lanes), waves)
+    else:
+        grid_x = ceil_div(items, nt)
+    D = dict(NT=nt, TH=th, TW=tw, NT_STORE=int(_special(special, "nt_store")[0]), SHFL=shfl,
              CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=a["stride"][0], PAD=pad,
              DIL=a["dilation"][0], FACT=a["factor"], CP=p, CQ=q)
     del ih_t
-    return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(items, nt), 1, 1),
+    return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
                        (nt, 1, 1),
                        [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
 

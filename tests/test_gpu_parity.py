@@ -70,11 +70,13 @@ def run_plan(key, configs, host_inputs):
     return out.cpu().numpy()
 
 
-def conv_cfgs(op_cfg, inline=None):
+def conv_cfgs(op_cfg, inline=None, special=None):
     g = None
-    if inline is not None:
+    if inline is not None or special is not None:
         g = {k: [] for k in KEYS}
-        g["inline"] = [inline]
+        g["inline"] = [inline if inline is not None else [1, 0]]
+        if special is not None:
+            g["special"] = special
     return Config([{k: [] for k in KEYS}, op_cfg], g)
 
 
@@ -275,6 +277,29 @@ def test_depthwise_vs_oracle(oracle, args, th, tw, waves):
     b_, co, p, q = ref.shape
     out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves)), [x, w])
     assert rel(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("args,th,waves", [
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 7, 4),       # 7 lanes per row, 63 lanes per wavefront
+    ((1, 5, 8, 12, 1, 3, 1, 1, 1), 4, 1),         # 3 lanes per row, last wavefront partly idle
+    ((3, 7, 16, 64, 1, 3, 1, 1, 1), 2, 2),        # 16 lanes per row
+    ((1, 3, 9, 20, 2, 3, 1, 1, 1), 3, 1),         # factor 2, ragged rows per lane
+])
+def test_depthwise_shuffled_halo_vs_oracle(oracle, args, th, waves):
+    """Halo columns taken from neighbouring lanes (DPP shifts) instead of loads."""
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
+    b_, co, p, q = ref.shape
+    for nt_store in (0, 1):
+        out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, 4, waves), special=[[nt_store], [1]]), [x, w])
+        assert rel(out, ref) <= TOL, nt_store
+    # borders: a constant image must give border sums with missing taps
+    ones = np.ones_like(x)
+    out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, 4, waves), special=[[0], [1]]), [ones, w])
+    assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
 
 
 def test_default_schedule_kernels_vs_oracle(oracle):

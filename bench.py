@@ -46,15 +46,28 @@ WORKLOADS = [
 HEADLINE = 1  # configs[1] of BASELINE.json
 
 
-def roofline(bound, dtype, ops, nbytes, ms):
+def measured_traffic(name):
+    """HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE /
+    WRITE_SIZE runs of the shipped tuned config scaled by a plain copy of known
+    size (flextensor_amd/tuned/hbm_traffic.json); None when not recorded."""
+    path = os.path.join(ROOT, "flextensor_amd", "tuned", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f)[name]["hbm_bytes_per_launch"]
+    except Exception:  # noqa: BLE001
+        return None
+
+
+def roofline(name, bound, dtype, ops, nbytes, ms):
     if bound == "hbm":
         achieved = nbytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBS, "traffic": None}
+                "frac": achieved / PEAK_HBM_GBS, "traffic": measured_traffic(name)}
     peak = PEAK_I8_TOPS if dtype == "i8" else PEAK_F32_TFLOPS
     achieved = ops / (ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": peak,
-            "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak, "traffic": None}
+            "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak,
+            "traffic": measured_traffic(name)}
 
 
 def gpu_workload(key, seed=0):
@@ -89,6 +102,24 @@ def kernel_ms(built, m, iters=None, warmup=20):
         probe = built.time(m.sets, warmup=warmup, iters=10)
         iters = int(min(max(TIMED_WINDOW_MS / max(probe, 1e-4), 20), 1000))
     return built.time(m.sets, warmup=warmup, iters=iters), metric
+
+
+def copy_yardstick(mib, iters):
+    """Time copy_f32 over `mib` MiB (read) + `mib` MiB (write)."""
+    import ctypes as ct
+    import torch
+    from flextensor_amd import runtime as rt
+    from flextensor_amd.plan import current_stream
+    from flextensor_amd.templates import gfx950
+    n = mib * (1 << 20) // 4
+    src = torch.ones(n, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    mod = rt.Module(rt.compile_to_code(gfx950.template_source("elementwise.hip"), []), "copy_f32")
+    ms = mod.time((8192,), (256,), [rt.ptr(src), rt.ptr(dst), ct.c_longlong(n)], warmup=3,
+                  iters=iters, stream=current_stream())
+    assert torch.equal(src[:1024], dst[:1024])
+    return {"workload": "copy_%dMiB" % mib, "ms": ms, "read_bytes": n * 4, "write_bytes": n * 4,
+            "GBps_read_plus_write": 2 * n * 4 / ms / 1e6}
 
 
 def cpu_baseline_for(name, key, ops, budget_s):
@@ -144,6 +175,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
+    ap.add_argument("--copy-mib", type=int, default=0,
+                    help="instead of a workload, run a plain device copy of this many MiB "
+                         "(bandwidth yardstick; calibrates FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--workload", default=None, choices=[w[0] for w in WORKLOADS],
                     help="time this configuration as the headline instead of configs[1] "
                          "(used to profile one kernel at a time)")
@@ -162,6 +196,9 @@ def main():
     torch.cuda.set_device(0)
     props = rt.device_props(0)
 
+    if args.copy_mib:
+        print(json.dumps(copy_yardstick(args.copy_mib, max(args.steps, 1))))
+        return
     headline = HEADLINE if args.workload is None else [w[0] for w in WORKLOADS].index(args.workload)
     name, key, ops, nbytes, bound, dtype = WORKLOADS[headline]
     if dtype == "i8":
@@ -185,7 +222,7 @@ def main():
     if not ok:
         raise RuntimeError("headline plan fails the correctness gate (metric %g)" % metric)
     k_ms, _ = kernel_ms(built, m)
-    roof = roofline(bound, dtype, ops, nbytes, k_ms)
+    roof = roofline(name, bound, dtype, ops, nbytes, k_ms)
     roof["kernel"] = plan.specs[-1].kernel
     roof["kernel_ms"] = k_ms
     built.close()
@@ -195,7 +232,7 @@ def main():
         for (wname, wkey, wops, wbytes, wbound, wdtype) in WORKLOADS:
             b, mm, pl = gpu_workload(wkey)
             ms, met = kernel_ms(b, mm)
-            r = roofline(wbound, wdtype, wops, wbytes, ms)
+            r = roofline(wname, wbound, wdtype, wops, wbytes, ms)
             entry = {"workload": wname, "ms": ms, "dtype": wdtype,
                      "throughput": wops / (ms * 1e-3) / 1e12,
                      "throughput_unit": "TOP/s" if wdtype == "i8" else "TFLOP/s",

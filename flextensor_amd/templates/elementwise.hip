@@ -3,6 +3,7 @@
 //   fill_zero_f32   zero-fill of a float buffer; precedes a split-K GEMM whose
 //                   partial sums meet in C with atomics (a kernel rather than
 //                   a memset call so that the launch sequence stays capturable)
+//   copy_f32        streaming copy (bandwidth yardstick, counter calibration)
 //   zero_pad2d_f32  P[b][c][h][w] = X[b][c][h-PAD][w-PAD] inside, 0 outside
 //                   (flextensor/nn/ops.py:83-117), used when the graph config
 //                   does not inline the padding into the convolution
@@ -18,6 +19,17 @@ void fill_zero_f32(float* __restrict__ p, int n)
         reinterpret_cast<f32x4*>(p)[i] = (f32x4)(0.0f);
     const int t = (n4 << 2) + blockIdx.x * 256 + threadIdx.x;
     if (t < n) p[t] = 0.0f;
+}
+
+/* plain streaming copy of n floats (n % 4 == 0): the yardstick for achievable
+ * HBM bandwidth and for scaling the profiler's FETCH_SIZE / WRITE_SIZE */
+extern "C" __global__ __launch_bounds__(256)
+void copy_f32(const float* __restrict__ src, float* __restrict__ dst, long long n)
+{
+    const long long n4 = n >> 2;
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride)
+        reinterpret_cast<f32x4*>(dst)[i] = reinterpret_cast<const f32x4*>(src)[i];
 }
 
 #ifdef FT_PADK

@@ -14,6 +14,13 @@
 //   STAGES      1 or 2 LDS buffers
 //   PD          prefetch distance: global loads of tile t+PD are in flight
 //               (in PD register sets) while tile t is multiplied
+//   FRAGPF      1: fragment-prefetch pipeline. Tile t+1 is written to LDS at
+//               the *start* of iteration t (its global loads were issued one
+//               iteration earlier), the operand fragments of the next k-step
+//               are read from LDS while the MFMAs of the current one run, and
+//               the first fragments of tile t+1 are read right after the one
+//               barrier of the iteration, so that the matrix cores have work
+//               immediately after every barrier (needs STAGES 2, PD 1)
 //   GROUP_M     tile-traversal group height (L2 locality)
 //   XCD_REMAP   1: consecutive logical tiles stay on one XCD
 //   PAD         LDS row padding in bytes (multiple of 16); -1 selects
@@ -40,6 +47,7 @@
 #define BK FT_BK
 #define STAGES FT_STAGES
 #define PD FT_PD
+#define FRAGPF FT_FRAGPF
 #define GROUP_M FT_GROUP_M
 #define XCD_REMAP FT_XCD_REMAP
 #define PAD FT_PAD
@@ -222,6 +230,59 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         }
     };
 
+#if FRAGPF
+    {
+        const int arow = wm * REP_M * MFMA + li;
+        const int brow = wn * REP_N * MFMA + li;
+        auto load_frags = [&](int buf, int kk, i32x4 (&fa)[REP_M], i32x4 (&fb)[REP_N]) {
+            const signed char* as = &As[buf][arow * SROW];
+            const signed char* bs = &Bs[buf][brow * SROW];
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+                fa[i] = *reinterpret_cast<const i32x4*>(as + i * MFMA * SROW + PCOL(arow + i * MFMA, kk + 16 * lg));
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+                fb[j] = *reinterpret_cast<const i32x4*>(bs + j * MFMA * SROW + PCOL(brow + j * MFMA, kk + 16 * lg));
+        };
+        i32x4 fa[REP_M], fb[REP_N];
+        load_global(0, 0);
+        store_lds(0, 0);
+        if (KT > 1) load_global(1, 0);
+        __syncthreads();
+        load_frags(0, 0, fa, fb);
+        for (int kt = 0; kt < KT; ++kt) {
+            const int cur = kt & 1;
+            if (kt + 1 < KT) {
+                store_lds(cur ^ 1, 0);                 /* tile kt+1, loaded during iteration kt-1 */
+                __builtin_amdgcn_sched_barrier(0);
+                if (kt + 2 < KT) load_global(kt + 2, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += MFMA_K) {
+                i32x4 na[REP_M], nb[REP_N];
+                if (kk + MFMA_K < BK) {
+                    load_frags(cur, kk + MFMA_K, na, nb);
+                } else {
+                    /* every wavefront has read tile kt and written tile kt+1 */
+                    __syncthreads();
+                    if (kt + 1 < KT) load_frags(cur ^ 1, 0, na, nb);
+                }
+#pragma unroll
+                for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+                    for (int j = 0; j < REP_N; ++j)
+                        acc[i][j] = MFMA_OP(fa[i], fb[j], acc[i][j]);
+                if (kk + MFMA_K < BK || kt + 1 < KT) {
+#pragma unroll
+                    for (int i = 0; i < REP_M; ++i) fa[i] = na[i];
+#pragma unroll
+                    for (int j = 0; j < REP_N; ++j) fb[j] = nb[j];
+                }
+            }
+        }
+    }
+#else
     /* tile t: global -> register set t % PD -> LDS buffer -> MFMA */
 #pragma unroll
     for (int p = 0; p < PD; ++p)
@@ -245,6 +306,8 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             }
         }
     }
+
+#endif
 
 #pragma unroll
     for (int i = 0; i < REP_M; ++i) {

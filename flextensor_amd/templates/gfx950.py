@@ -88,6 +88,7 @@ class GemmView(object):
         kind = op.kind
         self.kind = kind
         self.conv = None
+        self.groups = 1
         if kind == "gemm":
             if op.attrs.get("transposeA"):
                 raise NotImplementedError("transposeA is not on the tuned path")
@@ -102,8 +103,6 @@ class GemmView(object):
             self.dtype = "int8"
         elif kind == "conv2d_nchw":
             a = op.attrs
-            if a["groups"] != 1:
-                raise NotImplementedError("grouped conv2d is not on the tuned path")
             if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
                     or a["dilation"][0] != a["dilation"][1]:
                 raise NotImplementedError("anisotropic stride/padding/dilation")
@@ -112,18 +111,29 @@ class GemmView(object):
             s = op.reduce_axis[1].extent  # rw
             r = op.reduce_axis[2].extent  # rh
             _, _, h, w = a["in_shape"]
-            self.M, self.N, self.K = kout, b * p * q, c * r * s
+            groups = a["groups"]
+            # one GEMM per group: c is already the per-group channel count
+            self.M, self.N, self.K = kout // groups, b * p * q, c * r * s
             self.mode = 1
             self.dtype = "float32"
-            self.conv = dict(CB=b, CC=c, CH=h, CW=w, CR=r, CS=s, CSTR=a["stride"][0],
+            self.groups = groups
+            self.conv = dict(CB=b, CG=groups, CC=c * groups, CH=h, CW=w, CR=r, CS=s, CSTR=a["stride"][0],
                              CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
         else:
             raise InvalidConfig("operator kind %s has no GEMM view" % kind)
         # K as the kernels iterate it: fp32 pads the tail up to a multiple of
-        # 16 (int8: 64) with predicated zero loads; int8 needs K % 16 == 0.
+        # 16 (int8: 64) with zero-filling loads unless it already is a multiple
+        # of 8; int8 needs K % 16 == 0.
         if min(self.M, self.N, self.K) < 1:
             raise InvalidConfig("empty operator: M, N, K = %d, %d, %d" % (self.M, self.N, self.K))
-        self.KP = ceil_div(self.K, 64) * 64 if self.dtype == "int8" else ceil_div(self.K, 16) * 16
+        if self.dtype == "int8":
+            self.KP_options = [ceil_div(self.K, 64) * 64]
+        else:
+            self.KP_options = [ceil_div(self.K, 16) * 16]
+            if self.K % 8 == 0 and self.K % 16 != 0:
+                # e.g. K = 72: unpadded for 32x32x2 tiles of 8 or 72, padded to 80 for 16x16x4
+                self.KP_options.insert(0, self.K)
+        self.KP = self.KP_options[-1]
 
 
 F32_BK = (8, 16, 32, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
@@ -142,11 +152,16 @@ def _gemm_space(view):
     def keep(e):
         return e[2] in bks and e[0] <= max_split
 
-    rs = SplitSpace(3, view.KP, keep=keep)
+    rs = SplitSpace(3, view.KP_options[0], keep=keep)
+    for other in view.KP_options[1:]:
+        extra = SplitSpace(3, other, keep=keep)
+        rs.static_entities = rs.static_entities + extra.static_entities
+        rs._index = {tuple(e): i for i, e in enumerate(rs.static_entities)}
+        rs.size = len(rs.static_entities)
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
     space.add_subspace("xcd_remap", EnumSpace([[1, 0], [0, 0]] if i8 else [[1, 0], [0, 0], [1, 1], [0, 1]]),
@@ -190,8 +205,9 @@ SPECIAL_DEFAULTS = {
     "halo_shfl": [0],
 }
 
-# unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles)
-PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3)}
+# unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
+# depth 5 = two stages with the fragment-prefetch pipeline (int8 GEMM)
+PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1)}
 
 
 def special_knobs(kind):
@@ -230,7 +246,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE:
+    if depth not in PIPELINE or (depth == 5 and view.dtype != "int8"):
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
@@ -256,10 +272,11 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     nacc = rm * rn * (mfm * mfm // 64)
     if nacc > MAX_ACC_REGS:
         raise InvalidConfig("accumulators need %d registers per lane" % nacc)
-    if splitk * waves_k * kiters * bk != view.KP:
+    kp = splitk * waves_k * kiters * bk
+    if kp not in view.KP_options:
         raise InvalidConfig("reduce split does not multiply to K")
     nt = wm * wn * 64          # threads of one k-group
-    D = dict(M=view.M, N=view.N, K=view.K, KP=view.KP, MFMA=mfm, WAVES_M=wm, WAVES_N=wn, REP_M=rm,
+    D = dict(M=view.M, N=view.N, K=view.K, KP=kp, MFMA=mfm, WAVES_M=wm, WAVES_N=wn, REP_M=rm,
              REP_N=rn, BK=bk, STAGES=stages, GROUP_M=group_m, XCD_REMAP=xcd)
 
     if i8:
@@ -281,7 +298,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         lds = stages * (bm + bn) * (bk + max(pad, 0))
         if lds > LDS_BYTES:
             raise InvalidConfig("LDS tile needs %d bytes" % lds)
-        D.update(PAD=pad, PD=pd, NT_STORE=int(_special(special, "nt_store")[0]))
+        D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0,
+                 NT_STORE=int(_special(special, "nt_store")[0]))
         grid = (gm * gn, 1, 1)
         spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])
@@ -317,7 +335,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     eb = ceil_div((bn * bk) // bv, nt)
     if (ea * av + eb * bv) * pd > 160:
         raise InvalidConfig("global->LDS staging needs too many registers")
-    if max(view.M * view.K, view.K * view.N, view.M * view.N) * 4 >= 2 ** 31:
+    if max(view.M * view.K, view.K * view.N, view.M * view.N) * view.groups * 4 >= 2 ** 31:
         raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
     D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
     specs = []
@@ -333,11 +351,11 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     else:
         a_name, b_name = in_names[0], in_names[1]
     if splitk > 1:
-        nout = view.M * view.N
+        nout = view.M * view.N * view.groups
         specs.append(KernelSpec("elementwise.hip", "fill_zero_f32", {},
                                 (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
                                 [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
-    grid = (gm * gn * splitk, 1, 1)
+    grid = (gm * gn * splitk * view.groups, 1, 1)
     specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt * waves_k, 1, 1),
                             [("buf", a_name), ("buf", b_name), ("buf", out_name)]))
     return specs

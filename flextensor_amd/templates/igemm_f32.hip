@@ -10,7 +10,10 @@
 //   MODE 1  conv2d NCHW       A = weight [Kout][C*R*S], B = im2col gather of
 //                             the input with zero padding folded into the
 //                             load predicate, N = batch*OH*OW
-//                             (flextensor/nn/ops.py:83-117, 419-479)
+//                             (flextensor/nn/ops.py:83-117, 419-479).
+//                             Grouped convolution (CG groups) runs one GEMM
+//                             per group: M = Kout/CG, K = (C/CG)*R*S, and the
+//                             group index is one more grid factor.
 //
 // Knobs (set by the scheduler from a Config):
 //   MFMA            32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
@@ -118,7 +121,7 @@ typedef f32x4 acc_t;
 #endif
 #define TILES_M ((M + BM - 1) / BM)
 #define TILES_N ((N + BN - 1) / BN)
-/* KP = K rounded up to a multiple of 16; the host checks KP % (SPLITK*BK) == 0.
+/* KP = K, or K rounded up to a multiple of 16 when K % 8 != 0; the host checks KP % (SPLITK*BK) == 0.
  * When KP != K the tail is zero-filled by the load predicates. */
 #define KSPLIT_LEN (KP / SPLITK)
 #define KGROUP_LEN (KSPLIT_LEN / WAVES_K)
@@ -176,10 +179,10 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #else
 #define LOAD_B ld_f32
 #endif
-#define A_BYTES (M * K * 4)
 
 #if MODE == 1
 #define CB FT_CB
+#define CG FT_CG
 #define CC FT_CC
 #define CH FT_CH
 #define CW FT_CW
@@ -193,6 +196,7 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 /* conv geometry, all compile-time: input [CB][CC][CH][CW], kernel CR x CS,
  * stride CSTR, padding CPAD, dilation CDIL, output CP x CQ. */
 #define OHW (CP * CQ)
+#define A_BYTES (CG * M * K * 4)
 #define B_BYTES (CB * CC * CH * CW * 4)
 /* When an LDS tile spans whole kernel windows (BK % (CR*CS) == 0) every
  * gathered element keeps its tap (r, s) and its channel offset inside the
@@ -207,6 +211,8 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #error "conv mode gathers scalars: BV must be 1"
 #endif
 #else
+#define CG 1
+#define A_BYTES (M * K * 4)
 #define B_BYTES (K * N * 4)
 #endif
 
@@ -241,11 +247,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const int lg = lane / MFMA;   /* k group */
 
     /* ---- workgroup -> (split, tile_m, tile_n) ------------------------- */
-    const int nblk = TILES_M * TILES_N * SPLITK;
+    const int nblk = TILES_M * TILES_N * SPLITK * CG;
     int bid = blockIdx.x;
 #if XCD_REMAP
     if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
 #endif
+    const int gi = bid / (TILES_M * TILES_N * SPLITK);   /* convolution group */
+    bid = bid % (TILES_M * TILES_N * SPLITK);
     const int kz = bid / (TILES_M * TILES_N);
     const int r = bid % (TILES_M * TILES_N);
     const int grp = r / (GROUP_M * TILES_N);
@@ -286,7 +294,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         const int p = nn % OHW;
         px_h[e] = (p / CQ) * CSTR - CPAD;
         px_w[e] = (p % CQ) * CSTR - CPAD;
-        px_off[e] = b * (CC * CH * CW);
+        px_off[e] = b * (CC * CH * CW) + gi * ((CC / CG) * CH * CW);
     }
 #endif
 
@@ -306,7 +314,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         const int m = m0 + a_row[e];
         bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
         if (M % BM != 0) ok = ok && (m < M);
-        a_voff[e] = ok ? (unsigned)(m * K + a_col[e]) * 4u : OOB;
+        a_voff[e] = ok ? (unsigned)((gi * M + m) * K + a_col[e]) * 4u : OOB;
     }
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
@@ -498,7 +506,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if MODE == 1
             const int b = n / OHW;
             const int p = n % OHW;
-            const size_t cbase = (size_t)b * M * OHW + p;
+            const size_t cbase = ((size_t)b * (CG * M) + (size_t)gi * M) * OHW + p;
 #endif
 #pragma unroll
             for (int v = 0; v < NACC; ++v) {

@@ -148,6 +148,22 @@ def test_golden_conv_small():
             assert rel(out, GOLD[yname]) <= TOL, (wname, inline)
 
 
+def test_golden_conv_grouped_reference_case():
+    """The reference's own conv2d test case (flextensor/test/test_ops.py:85-115):
+    x [4,6,7,7], w [9,2,3,3], stride 2, padding 1, dilation 2, groups 3."""
+    x, w = GOLD["conv_g3_x"], GOLD["conv_g3_w"]
+    args = (4, 6, 7, 7, 9, 3, 2, 1, 2, 3)
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    key = key_of("conv2d", "t", args)
+    # per group: M = 3, N = 4*3*3 = 36, K = 2*9 = 18 -> 32
+    for cfg in ({}, gcfg(3, 36, 32, 1, 1, 1, 1, 16, 16), gcfg(3, 36, 32, 1, 1, 2, 1, 16, 16, sk=2, wk=1),
+                gcfg(3, 36, 32, 1, 1, 1, 1, 32, 8, sk=2, st=3)):
+        for inline in ([1, 0], [0, 0]):
+            out = run_plan(key, conv_cfgs(cfg, inline), [x, w])
+            assert out.shape == (4, 9, 3, 3)
+            assert rel(out, GOLD["conv_g3_y"]) <= TOL, (cfg, inline)
+
+
 def test_golden_depthwise_reference_case():
     # the reference's own case: x [4,6,7,7], w [6,3,3,3], stride 2, pad 1, dilation 2
     x, w = GOLD["dw_x"], GOLD["dw_w"]
@@ -218,6 +234,10 @@ def test_gemm_transpose_b_vs_oracle(oracle):
     (256, 512, 384, dict(wm=1, rm=4, wn=2, rn=2, mf=16, bk=128, st=1)),
     (136, 208, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64)),      # ragged everywhere, K tail
     (512, 256, 512, dict(wm=2, rm=4, wn=2, rn=4, mf=32, bk=128, gm=2, xcd=0)),
+    (512, 512, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=5)),      # fragment-prefetch pipeline
+    (200, 320, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, st=5)),       # same, ragged, one k-step per tile
+    (256, 64, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=64, st=5)),        # same, a single tile
+    (256, 768, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=4)),      # prefetch 3 tiles
 ])
 def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
     register(gemm_int8, "gemm", "gemm_int8", (M, K, N), "rocm", 0)
@@ -240,6 +260,9 @@ CONV_CASES = [
     ((1, 3, 32, 32, 16, 7, 2, 3, 1, 1), dict(wm=1, rm=1, wn=4, rn=1, mf=16, bk=16)),   # 7x7 s2 p3, K=147
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=16, bk=16, sk=3, wk=1, st=3)),
     ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=32, sk=2, wk=1, st=4)),
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72)),              # groups 4, whole windows
+    ((2, 24, 10, 10, 24, 3, 1, 1, 1, 24), dict(wm=1, rm=1, wn=1, rn=2, mf=16, bk=16)),             # groups = channels
+    ((1, 16, 14, 14, 32, 3, 2, 1, 1, 2), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=8, sk=3)),         # groups 2, split-K atomics
 ]
 
 
@@ -252,8 +275,9 @@ def test_conv2d_vs_oracle(oracle, args, kn):
     nb, c, h, wd, ko, ks, st, pd, dl, g = args
     ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
     assert ref.shape == bufs[-1].shape
-    M, N, K = ko, nb * ref.shape[2] * ref.shape[3], c * ks * ks
-    cfg = gcfg(M, N, ceil_div(K, 16) * 16, **kn)
+    M, N, K = ko // g, nb * ref.shape[2] * ref.shape[3], (c // g) * ks * ks
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    cfg = gcfg(M, N, kp, **kn)
     for inline in ([1, 0], [0, 0]):
         out = run_plan(key, conv_cfgs(cfg, inline), [x, w])
         assert rel(out, ref) <= TOL, inline

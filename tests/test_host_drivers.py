@@ -1,0 +1,81 @@
+"""The tuning drivers (optimize_*.py): key construction, log append and replay,
+with a host-side cost function instead of the GPU."""
+import argparse
+import json
+import os
+
+import numpy as np
+
+from flextensor_amd.optimize import common, optimize_conv2d, optimize_depthwise_conv2d, optimize_gemm
+from flextensor_amd.scheduler import schedule_with_config
+from flextensor_amd.task import TASK_TABLE
+from flextensor_amd.tuned import load, lookup
+from flextensor_amd.utils import Config
+
+
+def parse(argv):
+    p = argparse.ArgumentParser()
+    common.init_arg_parser(p)
+    return p.parse_args(argv)
+
+
+def test_arg_parser_has_reference_flags():
+    a = parse([])
+    for flag in ("from_", "to", "log", "test", "trials", "target", "device", "timeout", "parallel",
+                 "use_model", "method", "slevel", "rlevel", "force_inline", "host", "target_host",
+                 "device_key", "use_rpc", "fcompile", "port", "check"):
+        assert hasattr(a, flag), flag
+    assert a.target == "rocm" and a.method == "searching" and a.slevel == 4 and a.rlevel == 3
+
+
+def test_driver_keys_are_registered():
+    a = parse([])
+    for i, e in enumerate(optimize_gemm.SHAPES["baseline"] + optimize_gemm.SHAPES["int8"]):
+        task, trials = optimize_gemm.make_task(i, e, a)
+        assert task.key in TASK_TABLE and len(trials) == 1
+    mk = optimize_conv2d.make_task_for("baseline")
+    for i, s in enumerate(optimize_conv2d.SHAPES["baseline"]):
+        task, trials = mk(i, s, a)
+        assert task.key in TASK_TABLE and len(trials) == 2
+    mk = optimize_conv2d.make_task_for("yolo")
+    assert mk(3, optimize_conv2d.SHAPES["yolo"][3], a)[0].key in TASK_TABLE
+    for i, s in enumerate(optimize_depthwise_conv2d.SHAPES["baseline"] + optimize_depthwise_conv2d.SHAPES["mobile"]):
+        assert optimize_depthwise_conv2d.make_task(i, s, a)[0].key in TASK_TABLE
+
+
+def test_run_driver_appends_log_and_replays(tmp_path, monkeypatch):
+    np.random.seed(0)
+    log = str(tmp_path / "gemm.log")
+
+    def cost(task_key, cfg, op_pos, number):
+        s, _ = schedule_with_config(task_key, cfg, op_pos=op_pos)
+        return 1.0 + 1e-3 * s.specs[-1].grid[0]
+
+    import flextensor_amd.scheduler as sch
+    real = sch.schedule
+    monkeypatch.setattr(sch, "schedule", lambda *a, **k: real(*a, evaluator=cost, verbose=False,
+                                                               **{x: y for x, y in k.items()}))
+    monkeypatch.setattr(common, "evaluate", lambda *a, **k: 0.5)
+    args = parse(["--log", log, "--trials", "2", "--parallel", "2", "--warm_up", "1x4"])
+    common.run_driver(args, optimize_gemm.SHAPES["baseline"], optimize_gemm.make_task, "gemm")
+    entries = load(log)
+    key = "gemm_gemm_(1024, 1024, 1024)_rocm(0)"
+    assert list(entries) == [key]
+    cfg = entries[key]
+    assert isinstance(cfg, Config) and cfg.op_config_lst[0]["spatial"]
+    with open(log) as f:
+        lines = [l for l in f.read().splitlines() if l]
+    assert lines[0].startswith("# 0.5") and lines[1].startswith(key + ":")
+    json.loads(lines[1].split(":", 1)[1])
+    s, _ = schedule_with_config(key, cfg)
+    assert s.specs[-1].kernel == "igemm_f32"
+
+
+def test_shipped_tuned_log_replays_for_every_benchmark_task():
+    import __graft_entry__ as g
+    for key in g.BENCH_KEYS:
+        cfg = lookup(key)
+        assert cfg is not None, key
+        s, bufs = schedule_with_config(key, cfg)
+        assert s.specs and len(bufs) == 3
+    assert os.path.exists(os.path.join(os.path.dirname(common.__file__), "..", "tuned", "mi355x.log"))

@@ -19,6 +19,10 @@ class KernelPlan(object):
         self.specs = list(specs)
         # name -> (shape, dtype) of buffers the plan owns (e.g. a padded image)
         self.intermediates = dict(intermediates)
+        # name -> (shape, dtype) of zero-initialised workspaces the kernels declare
+        self.workspaces = {}
+        for spec in self.specs:
+            self.workspaces.update(getattr(spec, "workspace", {}))
         self.configs = configs
         # argument names of the caller's buffers, inputs..., output
         self.buf_names = ["in%d" % i for i in range(len(bufs) - 1)] + ["out"]
@@ -68,6 +72,8 @@ class BuiltPlan(object):
         self.scratch = {}
         for name, (shape, dtype) in plan.intermediates.items():
             self.scratch[name] = torch.empty(shape, dtype=_torch_dtype(dtype), device="cuda")
+        for name, (shape, dtype) in plan.workspaces.items():
+            self.scratch[name] = torch.zeros(shape, dtype=_torch_dtype(dtype), device="cuda")
 
     def attrs(self):
         return [m.attrs() for m in self.modules]

@@ -29,6 +29,7 @@ LDS_BYTES = 160 * 1024        # per workgroup on gfx950
 MAX_ACC_REGS = 256            # accumulation VGPRs per lane
 MAX_THREADS = 1024
 NUM_XCD = 8
+NUM_CUS = 256                 # compute units of one MI355X
 
 
 class InvalidConfig(ValueError):
@@ -57,7 +58,11 @@ class KernelSpec(object):
                  ("u32", value) for scalars
     """
 
-    def __init__(self, template, kernel, defines, grid, block, args, lds_bytes=0, note=""):
+    def __init__(self, template, kernel, defines, grid, block, args, lds_bytes=0, note="",
+                 workspace=None):
+        # name -> (shape, dtype) of zero-initialised device buffers the plan
+        # owns and the kernel leaves zeroed where it relies on zeros
+        self.workspace = dict(workspace or {})
         self.template = template
         self.kernel = kernel
         self.defines = dict(defines)
@@ -164,7 +169,7 @@ def _gemm_space(view):
     space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
-    space.add_subspace("xcd_remap", EnumSpace([[1, 0], [0, 0]] if i8 else [[1, 0], [0, 0], [1, 1], [0, 1]]),
+    space.add_subspace("xcd_remap", EnumSpace([[1, 0], [0, 0]] if i8 else [[1, 0], [0, 0], [1, 1], [0, 1], [1, 0, 1], [1, 0, 2]]),
                        "reorder")
     return space
 
@@ -250,8 +255,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
-    ro = list((config.get("reorder") or [[1, 0]])[0]) + [0]
-    xcd, in_wg = int(ro[0]), int(ro[1])
+    ro = list((config.get("reorder") or [[1, 0]])[0]) + [0, 0]
+    xcd, in_wg, stream_k = int(ro[0]), int(ro[1]), int(ro[2])
     i8 = view.dtype == "int8"
     waves_k = 1
     if in_wg and splitk > 1:
@@ -280,7 +285,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
              REP_N=rn, BK=bk, STAGES=stages, GROUP_M=group_m, XCD_REMAP=xcd)
 
     if i8:
-        if splitk != 1:
+        if splitk != 1 or stream_k:
             raise InvalidConfig("int8 GEMM does not split K across workgroups")
         mfma_k = 32 if mfm == 32 else 64
         if bk % mfma_k != 0:
@@ -355,9 +360,25 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         specs.append(KernelSpec("elementwise.hip", "fill_zero_f32", {},
                                 (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
                                 [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
-    grid = (gm * gn * splitk * view.groups, 1, 1)
-    specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt * waves_k, 1, 1),
-                            [("buf", a_name), ("buf", b_name), ("buf", out_name)]))
+    args = [("buf", a_name), ("buf", b_name), ("buf", out_name)]
+    workspace = {}
+    if stream_k:
+        # balanced K streaming: stream_k workgroups per compute unit share the
+        # (tile, k-tile) units evenly; see the template for the protocol
+        if stream_k < 0 or splitk != 1 or waves_k != 1:
+            raise InvalidConfig("K streaming excludes the other K splits")
+        units = gm * gn * view.groups * (kp // bk)
+        per = ceil_div(units, NUM_CUS * stream_k)
+        ngrid = ceil_div(units, per)
+        D.update(SK_PER=per)
+        grid = (ngrid, 1, 1)
+        workspace = {out_name + "_parts": ((ngrid * 2 * nt * nacc,), "float32"),
+                     out_name + "_count": ((gm * gn * view.groups,), "int32")}
+        args += [("buf", out_name + "_parts"), ("buf", out_name + "_count")]
+    else:
+        grid = (gm * gn * splitk * view.groups, 1, 1)
+    specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt * waves_k, 1, 1), args,
+                            workspace=workspace))
     return specs
 
 

@@ -30,6 +30,14 @@
 //                   WAVES_M*WAVES_N wavefronts each multiply their own K slice
 //                   through their own LDS tiles; the partial tiles are summed
 //                   through LDS at the end (no atomics, no zero fill)
+//   SK_PER          > 0: balanced K streaming. The work is cut into units of
+//                   one LDS tile step (output tile, k-tile); every workgroup
+//                   takes SK_PER consecutive units, so a workgroup may
+//                   finish one output tile, run whole tiles and begin a
+//                   third. A partly covered tile is written to a workspace
+//                   slot; the workgroup that arrives last at the tile's
+//                   counter sums the slots in a fixed order and stores the
+//                   tile (no waiting, no zero fill, deterministic)
 //   GROUP_M         tile-traversal group height (L2 locality)
 //   XCD_REMAP       1: consecutive logical tiles stay on one XCD
 //   APAD / BPAD     LDS row padding in floats; APAD = -1 selects an unpadded
@@ -66,6 +74,11 @@
 #define BPAD FT_BPAD
 #define AV FT_AV
 #define BV FT_BV
+#ifdef FT_SK_PER
+#define SK_PER FT_SK_PER
+#else
+#define SK_PER 0
+#endif
 
 #ifndef FT_MODE
 #error "FT_MODE must be defined"
@@ -223,7 +236,11 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 
 extern "C" __global__ __launch_bounds__(NTW)
 void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
-               float* __restrict__ C)
+               float* __restrict__ C
+#if SK_PER > 0
+               , float* sk_part, unsigned* sk_cnt
+#endif
+               )
 {
     __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
     /* k-group of this wavefront (NT is a multiple of 64, so it is uniform
@@ -246,26 +263,6 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const int li = lane % MFMA;   /* row (A) / column (B, C) inside an MFMA tile */
     const int lg = lane / MFMA;   /* k group */
 
-    /* ---- workgroup -> (split, tile_m, tile_n) ------------------------- */
-    const int nblk = TILES_M * TILES_N * SPLITK * CG;
-    int bid = blockIdx.x;
-#if XCD_REMAP
-    if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
-#endif
-    const int gi = bid / (TILES_M * TILES_N * SPLITK);   /* convolution group */
-    bid = bid % (TILES_M * TILES_N * SPLITK);
-    const int kz = bid / (TILES_M * TILES_N);
-    const int r = bid % (TILES_M * TILES_N);
-    const int grp = r / (GROUP_M * TILES_N);
-    const int first_m = grp * GROUP_M;
-    const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
-    const int rr = r % (GROUP_M * TILES_N);
-    const int tile_m = first_m + rr % gsz;
-    const int tile_n = rr / gsz;
-    const int m0 = tile_m * BM;
-    const int n0 = tile_n * BN;
-    const int kbase = kz * KSPLIT_LEN + kg * KGROUP_LEN;
-
     /* ---- per-thread load coordinates ----------------------------------- */
     int a_row[EA], a_col[EA];
 #pragma unroll
@@ -281,6 +278,53 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         b_row[e] = q / B_CHUNKS_ROW;
         b_col[e] = (q % B_CHUNKS_ROW) * BV;
     }
+    /* ---- workgroup -> (group, split, tile_m, tile_n) and K range -------- */
+#if SK_PER > 0
+#if SPLITK != 1 || WAVES_K != 1
+#error "balanced K streaming excludes the other K splits"
+#endif
+#define SK_UNITS (TILES_M * TILES_N * CG * KT)
+#define SK_GRID ((SK_UNITS + SK_PER - 1) / SK_PER)
+#define SK_SLOT (NT * REP_M * REP_N * NACC)
+    __shared__ unsigned sk_arrived;
+    int wg = blockIdx.x;
+#if XCD_REMAP
+    if (SK_GRID % 8 == 0) wg = (wg % 8) * (SK_GRID / 8) + wg / 8;
+#endif
+    int unit = wg * SK_PER;
+    const int unit_end = (unit + SK_PER < SK_UNITS) ? unit + SK_PER : SK_UNITS;
+    while (unit < unit_end) {
+    const int tile = unit / KT;
+    const int kt_lo = unit - tile * KT;
+    const int nk = (KT - kt_lo < unit_end - unit) ? KT - kt_lo : unit_end - unit;
+    unit += nk;
+    const int gi = tile / (TILES_M * TILES_N);
+    const int kz = 0;
+    const int r = tile % (TILES_M * TILES_N);
+#else
+    {
+    const int nblk = TILES_M * TILES_N * SPLITK * CG;
+    int bid = blockIdx.x;
+#if XCD_REMAP
+    if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
+#endif
+    const int gi = bid / (TILES_M * TILES_N * SPLITK);   /* convolution group */
+    bid = bid % (TILES_M * TILES_N * SPLITK);
+    const int kz = bid / (TILES_M * TILES_N);
+    const int r = bid % (TILES_M * TILES_N);
+    const int kt_lo = 0;
+    const int nk = KT;
+#endif
+    const int grp = r / (GROUP_M * TILES_N);
+    const int first_m = grp * GROUP_M;
+    const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
+    const int rr = r % (GROUP_M * TILES_N);
+    const int tile_m = first_m + rr % gsz;
+    const int tile_n = rr / gsz;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+    const int kbase = kz * KSPLIT_LEN + kg * KGROUP_LEN + kt_lo * BK;
+
 #if MODE == 1
     /* pixel decomposition of each column this thread gathers */
     int px_off[EB], px_h[EB], px_w[EB];
@@ -448,22 +492,22 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
      * flight; tile kt+1 is written to LDS right after the MFMAs of tile kt. */
 #pragma unroll
     for (int p = 0; p < PD; ++p)
-        if (p < KT) load_global(p, p);
+        if (p < nk) load_global(p, p);
     store_lds(0, 0);
     __syncthreads();
-    for (int kt0 = 0; kt0 < KT; kt0 += PD) {
+    for (int kt0 = 0; kt0 < nk; kt0 += PD) {
 #pragma unroll
         for (int u = 0; u < PD; ++u) {
             const int kt = kt0 + u;
-            if (kt < KT) {
+            if (kt < nk) {
                 const int cur = (STAGES == 2) ? (kt & 1) : 0;
-                if (kt + PD < KT) load_global(kt + PD, u);
+                if (kt + PD < nk) load_global(kt + PD, u);
                 /* keep the prefetch at the top of the iteration: without this
                  * fence the scheduler sinks the loads down to their use */
                 __builtin_amdgcn_sched_barrier(0);
                 compute(cur);
                 if (STAGES == 1) __syncthreads();
-                if (kt + 1 < KT) store_lds((STAGES == 2) ? (cur ^ 1) : 0, (u + 1) % PD);
+                if (kt + 1 < nk) store_lds((STAGES == 2) ? (cur ^ 1) : 0, (u + 1) % PD);
                 __syncthreads();
             }
         }
@@ -494,6 +538,56 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
                 for (int v = 0; v < NACC; ++v)
                     acc[i][j][v] += red[((i * REP_N + j) * NACC + v) * NT + tid];
+    }
+#endif
+
+#if SK_PER > 0
+    if (nk != KT) {
+        /* ---- a partly covered tile: park it, the last arrival sums -------- */
+        /* The workgroups that share a tile are consecutive. Each owns two
+         * slots: slot 0 for the tile its range begins in, slot 1 for the tile
+         * it ends in after beginning in an earlier one. */
+        const int tile_u0 = tile * KT;
+        const int wg_first = tile_u0 / SK_PER;
+        const int wg_last = (tile_u0 + KT - 1) / SK_PER;
+        float* mine = sk_part + (size_t)(2 * wg + ((wg * SK_PER >= tile_u0) ? 0 : 1)) * SK_SLOT;
+        /* Slots are written and read with device-scope atomic accesses: they
+         * are coherent across the per-XCD L2 caches by themselves, so no
+         * cache write-back or invalidation is needed, only ordering: every
+         * wavefront waits for its slot stores before the barrier, and the
+         * arrival count is taken after the barrier. */
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v)
+                    __hip_atomic_store(&mine[((i * REP_N + j) * NACC + v) * NT + tid], acc[i][j][v],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0) sk_arrived = atomicAdd(&sk_cnt[tile], 1u);
+        __syncthreads();
+        const unsigned before_me = sk_arrived;
+        __syncthreads();
+        if (before_me != (unsigned)(wg_last - wg_first)) continue;
+        if (tid == 0) atomicExch(&sk_cnt[tile], 0u);   /* ready for the next launch */
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+                acc[i][j] = (acc_t)(0.0f);
+        for (int w = wg_first; w <= wg_last; ++w) {
+            float* part = sk_part + (size_t)(2 * w + ((w * SK_PER >= tile_u0) ? 0 : 1)) * SK_SLOT;
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+                for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                    for (int v = 0; v < NACC; ++v)
+                        acc[i][j][v] += __hip_atomic_load(&part[((i * REP_N + j) * NACC + v) * NT + tid],
+                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 #endif
 
@@ -534,4 +628,5 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             }
         }
     }
+    }   /* tile / segment */
 }

@@ -119,6 +119,32 @@ def test_lowering_rejects_bad_configs():
         schedule_with_config(I8, Config([i8], None))
 
 
+def test_k_streaming_lowering():
+    """reorder [[xcd, 0, s]]: s workgroups per compute unit share the (tile, k-tile) units."""
+    cfg = _gemm_cfg([8, 2, 2, 32], [8, 2, 2, 32], [1, 32, 32])          # 64 tiles x 32 k-tiles
+    cfg["reorder"] = [[1, 0, 1]]
+    s, _ = schedule_with_config(GEMM, Config([cfg], None))
+    spec = s.specs[-1]
+    assert [x.kernel for x in s.specs] == ["igemm_f32"]                  # no zero fill
+    assert spec.defines["SK_PER"] == 8 and spec.grid == (256, 1, 1)      # 2048 units over 256 CUs
+    slot = 256 * 4 * 16                                                  # threads x accumulators
+    assert s.workspaces == {"out_parts": ((256 * 2 * slot,), "float32"), "out_count": ((64,), "int32")}
+    assert [a[1] for a in spec.args] == ["in0", "in1", "out", "out_parts", "out_count"]
+    cfg["reorder"] = [[1, 0, 2]]
+    s, _ = schedule_with_config(GEMM, Config([cfg], None))
+    assert s.specs[-1].defines["SK_PER"] == 4 and s.specs[-1].grid == (512, 1, 1)
+    # excluded together with the other K splits, and for int8
+    for rd, ro in (([2, 16, 32], [1, 0, 1]), ([2, 16, 32], [1, 1, 1])):
+        bad = _gemm_cfg([8, 2, 2, 32], [8, 2, 2, 32], rd)
+        bad["reorder"] = [ro]
+        with pytest.raises(gfx950.InvalidConfig):
+            schedule_with_config(GEMM, Config([bad], None))
+    i8 = _gemm_cfg([16, 2, 4, 32], [16, 2, 4, 32], [1, 64, 64])
+    i8["reorder"] = [[1, 0, 1]]
+    with pytest.raises(gfx950.InvalidConfig):
+        schedule_with_config(I8, Config([i8], None))
+
+
 def test_lds_budget_respected_over_whole_space():
     ops, _ = TASK_TABLE[I8].func(*TASK_TABLE[I8].args)
     op_lst, down = flatten_graph(ops)

@@ -83,7 +83,8 @@ def gpu_workload(key, seed=0):
     return built, m, s
 
 
-TIMED_WINDOW_MS = 2.5   # every workload is timed over about this much device time
+TIMED_WINDOW_MS = 25.0  # every workload is timed over about this much device time
+WARM_MS = 150.0         # untimed device work first: idle clocks need ~100 ms to reach steady state
 
 
 def kernel_ms(built, m, iters=None, warmup=20):
@@ -100,8 +101,8 @@ def kernel_ms(built, m, iters=None, warmup=20):
         raise RuntimeError("tuned plan fails the correctness gate (metric %g)" % metric)
     if iters is None:
         probe = built.time(m.sets, warmup=warmup, iters=10)
-        iters = int(min(max(TIMED_WINDOW_MS / max(probe, 1e-4), 20), 1000))
-    return built.time(m.sets, warmup=warmup, iters=iters), metric
+        iters = int(min(max(TIMED_WINDOW_MS / max(probe, 1e-4), 20), 10000))
+    return built.time(m.sets, warmup=warmup, iters=iters, warm_ms=WARM_MS), metric
 
 
 def copy_yardstick(mib, iters):
@@ -170,8 +171,11 @@ def cpu_baseline_for(name, key, ops, budget_s):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps K (default: about %g ms of device time)" % TIMED_WINDOW_MS)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps W (default: about %g ms of device time, which is what "
+                         "idle clocks need to reach their steady state)" % WARM_MS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
@@ -197,18 +201,24 @@ def main():
     props = rt.device_props(0)
 
     if args.copy_mib:
-        print(json.dumps(copy_yardstick(args.copy_mib, max(args.steps, 1))))
+        print(json.dumps(copy_yardstick(args.copy_mib, max(args.steps or 100, 1))))
         return
     headline = HEADLINE if args.workload is None else [w[0] for w in WORKLOADS].index(args.workload)
     name, key, ops, nbytes, bound, dtype = WORKLOADS[headline]
-    if dtype == "i8":
-        args.steps = min(args.steps, 100)
     built, m, plan = gpu_workload(key)
     # ---- headline: W untimed steps, exactly K timed steps -----------------
     launches = built.launches(m.sets[0])
     stream = current_stream()
-    for _ in range(args.warmup):
-        rt.launch_seq(launches, stream=stream)
+    if args.steps is None or args.warmup is None:
+        probe = built.time(m.sets, warmup=5, iters=20)
+        if args.steps is None:
+            args.steps = int(min(max(TIMED_WINDOW_MS / probe, 100), 100000))
+        if args.warmup is None:
+            args.warmup = int(min(max(WARM_MS / probe, 100), 100000))
+    if args.warmup > 0:
+        wseq = launches * args.warmup
+        rt._check(rt.lib().ftr_launch_seq(rt._desc_array(wseq), len(wseq), ctypes.c_void_p(stream)),
+                  "ftr_launch_seq")
     torch.cuda.synchronize()
     seq = launches * args.steps          # one C call enqueues all K steps
     arr = rt._desc_array(seq)

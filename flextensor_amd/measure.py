@@ -25,6 +25,7 @@ from .templates import gfx950
 from .utils import to_tuple, ceil_div
 
 FP32_TOL = 1e-5
+WARM_MS = 60.0             # untimed device work before a candidate is timed
 # buffers of a memory-bound operator are rotated so that consecutive timed
 # launches do not find their data in the 256 MB last-level cache
 LLC_BYTES = 256 << 20
@@ -177,8 +178,10 @@ class Measurer(object):
         torch.cuda.synchronize()
         return ok, metric
 
-    def evaluate(self, plan, number=10, warmup=2):
-        """ms per run of ``plan``; raises on build failure or wrong output."""
+    def evaluate(self, plan, number=10, warmup=2, warm_ms=WARM_MS):
+        """ms per run of ``plan``; raises on build failure or wrong output.
+        Candidates are compiled between measurements, so each one meets an
+        idle device: ``warm_ms`` of untimed runs bring the clocks up first."""
         import torch
         built = plan.build()
         try:
@@ -189,7 +192,7 @@ class Measurer(object):
             ok, metric = self.check(first[-1])
             if not ok:
                 raise WrongResult("output differs from the default schedule (metric %g)" % metric)
-            return built.time(self.sets, warmup=warmup, iters=max(int(number), 1))
+            return built.time(self.sets, warmup=warmup, iters=max(int(number), 1), warm_ms=warm_ms)
         finally:
             built.close()
 

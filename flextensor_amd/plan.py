@@ -116,10 +116,19 @@ class BuiltPlan(object):
     def __call__(self, *tensors):
         rt.launch_seq(self.launches(tensors), stream=current_stream())
 
-    def time(self, tensor_sets, warmup=2, iters=10):
-        """Mean ms per run, rotating through ``tensor_sets``."""
+    def time(self, tensor_sets, warmup=2, iters=10, warm_ms=0.0):
+        """Mean ms per run, rotating through ``tensor_sets``.
+
+        ``warm_ms`` > 0 keeps the device busy with untimed runs for about that
+        long first: after an idle period the clocks take on the order of
+        100 ms of continuous work to reach their steady state, and a kernel
+        timed before that reads 15-25 % slow."""
         sets = [self.launches(ts) for ts in tensor_sets]
-        return rt.time_seq(sets, warmup=warmup, iters=iters, stream=current_stream())
+        stream = current_stream()
+        if warm_ms > 0:
+            probe = rt.time_seq(sets, warmup=1, iters=3, stream=stream)
+            warmup = max(warmup, int(min(warm_ms / max(probe, 1e-4), 1e6)))
+        return rt.time_seq(sets, warmup=warmup, iters=iters, stream=stream)
 
     def close(self):
         for m in self.modules:

@@ -279,6 +279,55 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         b_col[e] = (q % B_CHUNKS_ROW) * BV;
     }
     /* ---- workgroup -> (group, split, tile_m, tile_n) and K range -------- */
+    /* tile index inside one group -> first row / column of the tile */
+    auto tile_origin = [&](int r, int& m0_, int& n0_) {
+        const int grp = r / (GROUP_M * TILES_N);
+        const int first_m = grp * GROUP_M;
+        const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
+        const int rr = r % (GROUP_M * TILES_N);
+        m0_ = (first_m + rr % gsz) * BM;
+        n0_ = (rr / gsz) * BN;
+    };
+    acc_t acc[REP_M][REP_N];
+    /* accumulators -> C for the tile at (m0_, n0_) of group gi_ */
+    auto store_c = [&](int m0_, int n0_, int gi_) {
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i) {
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j) {
+                const int n = n0_ + (wn * REP_N + j) * MFMA + li;
+#if MODE == 1
+                const int b = n / OHW;
+                const int p = n % OHW;
+                const size_t cbase = ((size_t)b * (CG * M) + (size_t)gi_ * M) * OHW + p;
+#endif
+#pragma unroll
+                for (int v = 0; v < NACC; ++v) {
+#if MFMA == 32
+                    const int row = 8 * (v / 4) + 4 * lg + (v % 4);
+#else
+                    const int row = 4 * lg + v;
+#endif
+                    const int m = m0_ + (wm * REP_M + i) * MFMA + row;
+                    bool ok = true;
+                    if (M % BM != 0) ok = ok && (m < M);
+                    if (N % BN != 0) ok = ok && (n < N);
+                    if (ok) {
+#if MODE == 1
+                        float* dst = C + cbase + (size_t)m * OHW;
+#else
+                        float* dst = C + (size_t)m * N + n;
+#endif
+#if SPLITK > 1
+                        unsafeAtomicAdd(dst, acc[i][j][v]);
+#else
+                        *dst = acc[i][j][v];
+#endif
+                    }
+                }
+            }
+        }
+    };
 #if SK_PER > 0
 #if SPLITK != 1 || WAVES_K != 1
 #error "balanced K streaming excludes the other K splits"
@@ -286,13 +335,53 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #define SK_UNITS (TILES_M * TILES_N * CG * KT)
 #define SK_GRID ((SK_UNITS + SK_PER - 1) / SK_PER)
 #define SK_SLOT (NT * REP_M * REP_N * NACC)
+    /* A tile that several workgroups cover is exchanged through workspace
+     * slots. The sharers of a tile are consecutive workgroups; each owns two
+     * slots: slot 0 for the tile its range begins in, slot 1 for the tile it
+     * ends in after beginning in an earlier one. Slots are written and read
+     * with device-scope atomic accesses: these are coherent across the
+     * per-XCD L2 caches by themselves, so no cache write-back or invalidation
+     * is needed, only ordering: a wavefront waits for its slot stores before
+     * the barrier that precedes the arrival count. Nobody waits for anybody:
+     * whoever finds all other sharers arrived sums the slots, always in
+     * sharer order, so the result does not depend on the timing. */
     __shared__ unsigned sk_arrived;
+    auto sharers = [&](int tile_, int& first_, int& last_) {
+        first_ = (tile_ * KT) / SK_PER;
+        last_ = (tile_ * KT + KT - 1) / SK_PER;
+    };
+    auto slot_of = [&](int w, int tile_) -> float* {
+        return sk_part + (size_t)(2 * w + ((w * SK_PER >= tile_ * KT) ? 0 : 1)) * SK_SLOT;
+    };
+    auto add_slots = [&](int tile_, int from, int to) {
+        for (int w = from; w <= to; ++w) {
+            float* part = slot_of(w, tile_);
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+                for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                    for (int v = 0; v < NACC; ++v)
+                        acc[i][j][v] += __hip_atomic_load(&part[((i * REP_N + j) * NACC + v) * NT + tid],
+                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+                acc[i][j] = (acc_t)(0.0f);
+    };
     int wg = blockIdx.x;
 #if XCD_REMAP
     if (SK_GRID % 8 == 0) wg = (wg % 8) * (SK_GRID / 8) + wg / 8;
 #endif
     int unit = wg * SK_PER;
     const int unit_end = (unit + SK_PER < SK_UNITS) ? unit + SK_PER : SK_UNITS;
+    int arrive_tile = -1;        /* slot written, arrival still to be counted */
+    int check_tile = -1;         /* arrival counted, result still to be looked at */
+    unsigned check_before = 0;   /* thread 0: sharers that had arrived before */
     while (unit < unit_end) {
     const int tile = unit / KT;
     const int kt_lo = unit - tile * KT;
@@ -315,14 +404,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const int kt_lo = 0;
     const int nk = KT;
 #endif
-    const int grp = r / (GROUP_M * TILES_N);
-    const int first_m = grp * GROUP_M;
-    const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
-    const int rr = r % (GROUP_M * TILES_N);
-    const int tile_m = first_m + rr % gsz;
-    const int tile_n = rr / gsz;
-    const int m0 = tile_m * BM;
-    const int n0 = tile_n * BN;
+    int m0, n0;
+    tile_origin(r, m0, n0);
     const int kbase = kz * KSPLIT_LEN + kg * KGROUP_LEN + kt_lo * BK;
 
 #if MODE == 1
@@ -439,7 +522,6 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         }
     };
 
-    acc_t acc[REP_M][REP_N];
 #pragma unroll
     for (int i = 0; i < REP_M; ++i)
 #pragma unroll
@@ -494,7 +576,20 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     for (int p = 0; p < PD; ++p)
         if (p < nk) load_global(p, p);
     store_lds(0, 0);
+#if SK_PER > 0
+    /* The arrival for the slot written at the end of the previous segment is
+     * counted here: the wait for this tile's first loads has covered the slot
+     * stores, so the exchange costs this segment nothing. */
+    if (arrive_tile >= 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+#endif
     __syncthreads();
+#if SK_PER > 0
+    if (arrive_tile >= 0) {
+        if (tid == 0) check_before = atomicAdd(&sk_cnt[arrive_tile], 1u);
+        check_tile = arrive_tile;
+        arrive_tile = -1;
+    }
+#endif
     for (int kt0 = 0; kt0 < nk; kt0 += PD) {
 #pragma unroll
         for (int u = 0; u < PD; ++u) {
@@ -543,19 +638,26 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 
 #if SK_PER > 0
     if (nk != KT) {
-        /* ---- a partly covered tile: park it, the last arrival sums -------- */
-        /* The workgroups that share a tile are consecutive. Each owns two
-         * slots: slot 0 for the tile its range begins in, slot 1 for the tile
-         * it ends in after beginning in an earlier one. */
-        const int tile_u0 = tile * KT;
-        const int wg_first = tile_u0 / SK_PER;
-        const int wg_last = (tile_u0 + KT - 1) / SK_PER;
-        float* mine = sk_part + (size_t)(2 * wg + ((wg * SK_PER >= tile_u0) ? 0 : 1)) * SK_SLOT;
-        /* Slots are written and read with device-scope atomic accesses: they
-         * are coherent across the per-XCD L2 caches by themselves, so no
-         * cache write-back or invalidation is needed, only ordering: every
-         * wavefront waits for its slot stores before the barrier, and the
-         * arrival count is taken after the barrier. */
+        int wg_first, wg_last;
+        sharers(tile, wg_first, wg_last);
+        const unsigned others = (unsigned)(wg_last - wg_first);
+        if (kt_lo == 0) {
+            /* this workgroup holds the lowest K range and ends its run here,
+             * long after the other sharers began theirs: when all of them
+             * have arrived, add their slots to the registers and store */
+            if (tid == 0)
+                sk_arrived = __hip_atomic_load(&sk_cnt[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            const bool all_in = (sk_arrived == others);
+            __syncthreads();
+            if (all_in) {
+                add_slots(tile, wg_first + 1, wg_last);
+                if (tid == 0) atomicExch(&sk_cnt[tile], 0u);   /* ready for the next launch */
+                store_c(m0, n0, gi);
+                continue;
+            }
+        }
+        float* mine = slot_of(wg, tile);
 #pragma unroll
         for (int i = 0; i < REP_M; ++i)
 #pragma unroll
@@ -564,69 +666,40 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                 for (int v = 0; v < NACC; ++v)
                     __hip_atomic_store(&mine[((i * REP_N + j) * NACC + v) * NT + tid], acc[i][j][v],
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (unit < unit_end) {
+            arrive_tile = tile;      /* counted in the next segment's prologue */
+            continue;
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0) sk_arrived = atomicAdd(&sk_cnt[tile], 1u);
         __syncthreads();
         const unsigned before_me = sk_arrived;
         __syncthreads();
-        if (before_me != (unsigned)(wg_last - wg_first)) continue;
-        if (tid == 0) atomicExch(&sk_cnt[tile], 0u);   /* ready for the next launch */
-#pragma unroll
-        for (int i = 0; i < REP_M; ++i)
-#pragma unroll
-            for (int j = 0; j < REP_N; ++j)
-                acc[i][j] = (acc_t)(0.0f);
-        for (int w = wg_first; w <= wg_last; ++w) {
-            float* part = sk_part + (size_t)(2 * w + ((w * SK_PER >= tile_u0) ? 0 : 1)) * SK_SLOT;
-#pragma unroll
-            for (int i = 0; i < REP_M; ++i)
-#pragma unroll
-                for (int j = 0; j < REP_N; ++j)
-#pragma unroll
-                    for (int v = 0; v < NACC; ++v)
-                        acc[i][j][v] += __hip_atomic_load(&part[((i * REP_N + j) * NACC + v) * NT + tid],
-                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (before_me != others) continue;
+        if (tid == 0) atomicExch(&sk_cnt[tile], 0u);
+        clear_acc();
+        add_slots(tile, wg_first, wg_last);
     }
 #endif
-
-    /* ---- epilogue: accumulators -> C ----------------------------------- */
-#pragma unroll
-    for (int i = 0; i < REP_M; ++i) {
-#pragma unroll
-        for (int j = 0; j < REP_N; ++j) {
-            const int n = n0 + (wn * REP_N + j) * MFMA + li;
-#if MODE == 1
-            const int b = n / OHW;
-            const int p = n % OHW;
-            const size_t cbase = ((size_t)b * (CG * M) + (size_t)gi * M) * OHW + p;
-#endif
-#pragma unroll
-            for (int v = 0; v < NACC; ++v) {
-#if MFMA == 32
-                const int row = 8 * (v / 4) + 4 * lg + (v % 4);
-#else
-                const int row = 4 * lg + v;
-#endif
-                const int m = m0 + (wm * REP_M + i) * MFMA + row;
-                bool ok = true;
-                if (M % BM != 0) ok = ok && (m < M);
-                if (N % BN != 0) ok = ok && (n < N);
-                if (ok) {
-#if MODE == 1
-                    float* dst = C + cbase + (size_t)m * OHW;
-#else
-                    float* dst = C + (size_t)m * N + n;
-#endif
-#if SPLITK > 1
-                    unsafeAtomicAdd(dst, acc[i][j][v]);
-#else
-                    *dst = acc[i][j][v];
-#endif
-                }
-            }
-        }
-    }
+    store_c(m0, n0, gi);
     }   /* tile / segment */
+#if SK_PER > 0
+    if (check_tile >= 0) {
+        /* the first segment's arrival: if every other sharer had arrived
+         * before, the sum falls to this workgroup */
+        if (tid == 0) sk_arrived = check_before;
+        __syncthreads();
+        int wg_first, wg_last;
+        sharers(check_tile, wg_first, wg_last);
+        if (sk_arrived == (unsigned)(wg_last - wg_first)) {
+            if (tid == 0) atomicExch(&sk_cnt[check_tile], 0u);
+            clear_acc();
+            add_slots(check_tile, wg_first, wg_last);
+            int m0, n0;
+            tile_origin(check_tile % (TILES_M * TILES_N), m0, n0);
+            store_c(m0, n0, check_tile / (TILES_M * TILES_N));
+        }
+    }
+#endif
 }

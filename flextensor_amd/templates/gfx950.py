@@ -333,6 +333,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     else:
         lds_b = bk * (bn + bpad)
     lds = max(waves_k * stages * 4 * (bm * sa + lds_b), (waves_k - 1) * nt * nacc * 4)
+    if stream_k:
+        lds += 16             # the arrival word of the K-streaming exchange
     if lds > LDS_BYTES:
         raise InvalidConfig("LDS tile needs %d bytes" % lds)
     # staging registers for the global->LDS copy must stay reasonable
@@ -370,6 +372,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         units = gm * gn * view.groups * (kp // bk)
         per = ceil_div(units, NUM_CUS * stream_k)
         ngrid = ceil_div(units, per)
+        if xcd:
+            ngrid = ceil_div(ngrid, NUM_XCD) * NUM_XCD   # renumbering by XCD needs whole rounds
         D.update(SK_PER=per)
         grid = (ngrid, 1, 1)
         workspace = {out_name + "_parts": ((ngrid * 2 * nt * nacc,), "float32"),

@@ -333,7 +333,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #error "balanced K streaming excludes the other K splits"
 #endif
 #define SK_UNITS (TILES_M * TILES_N * CG * KT)
+/* the grid is rounded up to a multiple of 8 when workgroups are renumbered by
+ * XCD; the extra workgroups find no units */
+#if XCD_REMAP
+#define SK_GRID ((((SK_UNITS + SK_PER - 1) / SK_PER) + 7) / 8 * 8)
+#else
 #define SK_GRID ((SK_UNITS + SK_PER - 1) / SK_PER)
+#endif
 #define SK_SLOT (NT * REP_M * REP_N * NACC)
     /* A tile that several workgroups cover is exchanged through workspace
      * slots. The sharers of a tile are consecutive workgroups; each owns two
@@ -375,7 +381,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     };
     int wg = blockIdx.x;
 #if XCD_REMAP
-    if (SK_GRID % 8 == 0) wg = (wg % 8) * (SK_GRID / 8) + wg / 8;
+    wg = (wg % 8) * (SK_GRID / 8) + wg / 8;
 #endif
     int unit = wg * SK_PER;
     const int unit_end = (unit + SK_PER < SK_UNITS) ? unit + SK_PER : SK_UNITS;

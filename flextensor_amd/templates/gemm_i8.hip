@@ -26,6 +26,9 @@
 //   PAD         LDS row padding in bytes (multiple of 16); -1 selects
 //               unpadded rows whose 16-byte chunks are XOR-swizzled by row
 //   NT_STORE    1: non-temporal stores for C
+//   CVEC        1: the MFMA operands are swapped (the core computes the
+//               transposed tile), so a lane holds four consecutive columns of
+//               one row of C and writes them with one 128-bit store
 //
 // Both operands live in LDS as [rows][BK+PAD] bytes and are read as one
 // 128-bit load per lane per MFMA: lane (i, g) takes the 16 bytes at
@@ -52,6 +55,11 @@
 #define XCD_REMAP FT_XCD_REMAP
 #define PAD FT_PAD
 #define NT_STORE FT_NT_STORE
+#ifdef FT_CVEC
+#define CVEC FT_CVEC
+#else
+#define CVEC 0
+#endif
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
@@ -60,14 +68,19 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef i32x16 acc_t;
 #define NACC 16
 #define MFMA_K 32
-#define MFMA_OP(a, b, c) __builtin_amdgcn_mfma_i32_32x32x32_i8((a), (b), (c), 0, 0, 0)
+#define MFMA_RAW(a, b, c) __builtin_amdgcn_mfma_i32_32x32x32_i8((a), (b), (c), 0, 0, 0)
 #elif MFMA == 16
 typedef i32x4 acc_t;
 #define NACC 4
 #define MFMA_K 64
-#define MFMA_OP(a, b, c) __builtin_amdgcn_mfma_i32_16x16x64_i8((a), (b), (c), 0, 0, 0)
+#define MFMA_RAW(a, b, c) __builtin_amdgcn_mfma_i32_16x16x64_i8((a), (b), (c), 0, 0, 0)
 #else
 #error "MFMA must be 16 or 32"
+#endif
+#if CVEC
+#define MFMA_OP(a, b, c) MFMA_RAW((b), (a), (c))   /* rows of the result follow B's rows (n) */
+#else
+#define MFMA_OP(a, b, c) MFMA_RAW((a), (b), (c))
 #endif
 
 #define BM (WAVES_M * REP_M * MFMA)
@@ -309,6 +322,39 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
 
 #endif
 
+#if CVEC
+    /* swapped operands: lane (li, lg) holds C[m = li][n = 4*lg + 0..3] (16x16),
+     * or C[m = li][n = 8*q + 4*lg + 0..3] in registers 4q..4q+3 (32x32) */
+#pragma unroll
+    for (int i = 0; i < REP_M; ++i) {
+        const int m = m0 + (wm * REP_M + i) * MFMA + li;
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j) {
+#pragma unroll
+            for (int q = 0; q < NACC / 4; ++q) {
+#if MFMA == 32
+                const int n = n0 + (wn * REP_N + j) * MFMA + 8 * q + 4 * lg;
+#else
+                const int n = n0 + (wn * REP_N + j) * MFMA + 4 * lg;
+#endif
+                bool ok = true;
+                if (M % BM != 0) ok = ok && (m < M);
+                if (N % BN != 0) ok = ok && (n < N);      /* N % 4 == 0: whole vectors */
+                if (ok) {
+                    i32x4 v4;
+                    v4[0] = acc[i][j][4 * q + 0]; v4[1] = acc[i][j][4 * q + 1];
+                    v4[2] = acc[i][j][4 * q + 2]; v4[3] = acc[i][j][4 * q + 3];
+                    i32x4* dst = reinterpret_cast<i32x4*>(C + (size_t)m * N + n);
+#if NT_STORE
+                    __builtin_nontemporal_store(v4, dst);
+#else
+                    *dst = v4;
+#endif
+                }
+            }
+        }
+    }
+#else
 #pragma unroll
     for (int i = 0; i < REP_M; ++i) {
 #pragma unroll
@@ -335,4 +381,5 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             }
         }
     }
+#endif
 }

@@ -221,7 +221,7 @@ def special_knobs(kind):
     if kind in ("gemm", "conv2d_nchw"):
         return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
-        return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1]]}
+        return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1]], "halo_shfl": [[0], [1]]}
     return {}
@@ -303,8 +303,13 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         lds = stages * (bm + bn) * (bk + max(pad, 0))
         if lds > LDS_BYTES:
             raise InvalidConfig("LDS tile needs %d bytes" % lds)
-        D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0,
-                 NT_STORE=int(_special(special, "nt_store")[0]))
+        # nt_store: bit 0 = non-temporal stores, bit 1 = transposed MFMA so that lanes store 128-bit rows
+        store_mode = int(_special(special, "nt_store")[0])
+        if store_mode & 2 and view.N % 4 != 0:
+            raise InvalidConfig("128-bit C stores need N to be a multiple of 4")
+        D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0, NT_STORE=store_mode & 1)
+        if store_mode & 2:
+            D.update(CVEC=1)
         grid = (gm * gn, 1, 1)
         spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])

@@ -270,12 +270,32 @@ def test_gemm_transpose_b_vs_oracle(oracle):
     (256, 768, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=4)),      # prefetch 3 tiles
 ])
 def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
+    _gemm_int8_case(oracle, M, K, N, kn, None)
+
+
+@pytest.mark.parametrize("M,K,N,kn,store", [
+    (136, 208, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64), 2),           # 128-bit row stores, ragged
+    (200, 320, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, st=5), 2),
+    (256, 512, 384, dict(wm=1, rm=4, wn=2, rn=2, mf=16, bk=128), 3),         # same, non-temporal
+    (512, 256, 512, dict(wm=2, rm=4, wn=2, rn=4, mf=32, bk=128, gm=2), 3),
+])
+def test_gemm_int8_row_vector_stores(oracle, M, K, N, kn, store):
+    """nt_store bit 1: the MFMA computes the transposed tile so that a lane
+    holds four consecutive columns of one row."""
+    _gemm_int8_case(oracle, M, K, N, kn, store)
+
+
+def _gemm_int8_case(oracle, M, K, N, kn, store):
     register(gemm_int8, "gemm", "gemm_int8", (M, K, N), "rocm", 0)
     key = key_of("gemm", "gemm_int8", (M, K, N))
     _, bufs = TASK_TABLE[key].func(M, K, N)
     a, b = seeded_inputs(bufs, seed=K)
     assert a.min() == -128 and a.max() == 127
-    out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], None), [a, b])
+    g = None
+    if store is not None:
+        g = {k: [] for k in KEYS}
+        g["inline"], g["special"] = [[0]], [[-1, 0], [store]]
+    out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], g), [a, b])
     assert np.array_equal(out, oracle.gemm_i8_c(a, b))
     assert np.array_equal(out, oracle.gemm_i8_np(a, b))
 

@@ -182,6 +182,32 @@ class Scheduler(object):
         if self.verbose:
             print(*args, flush=True)
 
+    # ---- cost of a list of points: the device, or the ranking model -----
+    def _cost(self, configs, indices_lst, use_model=False):
+        """ms per point measured on the device, or (``use_model``) the ranking
+        network's scores, which order points but are not times
+        (flextensor/scheduler.py:239-243, 466-471)."""
+        if use_model:
+            return self.walker_group.query_performance(indices_lst)
+        next_configs = [self.walker_group.to_config(indices) for indices in indices_lst]
+        results = self.parallel_evaluate(configs, next_configs, number=self.number)
+        self.walker_group.add_perf_data(indices_lst, results)
+        return results
+
+    def _finish_with_model(self, configs, use_model):
+        """After a search driven by the ranking model, measure its best points
+        on the device and keep the measured order, so that what is returned is
+        a checked, timed kernel."""
+        if not use_model:
+            return
+        indices_lst = self.walker_group.topk(self.re_evalutate_number, modify=True)
+        self.walker_group.memory, self.walker_group.mem_size = [], 0
+        results = self._cost(configs, indices_lst, use_model=False)
+        self._log("measured after model search [ %s]" % "".join("%.6f " % r for r in results))
+        for indices, result in zip(indices_lst, results):
+            if result < float("inf"):
+                self.walker_group.record(indices, result, random_reject=False)
+
     # ---- warm-up: random points ---------------------------------------
     def _warm_up(self, warm_up_epoches, warm_up_trials, configs, type_keys, max_repeat=20,
                  use_model=False):
@@ -211,9 +237,7 @@ class Scheduler(object):
                     if k not in seen:
                         seen.add(k)
                         uniq.append(i)
-                results = self.parallel_evaluate(configs, [warm_up_configs[i] for i in uniq],
-                                                 number=self.number)
-                self.walker_group.add_perf_data([warm_up_indices[i] for i in uniq], results)
+                results = self._cost(configs, [warm_up_indices[i] for i in uniq], use_model)
                 self._log("warm up [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
                 for i, res in zip(uniq, results):
                     if res < float("inf"):
@@ -281,12 +305,105 @@ class Scheduler(object):
                 self.walker_group.visit.add(str(indices))
 
     def _random_schedule(self, configs, type_keys, use_model=False):
+        if use_model:
+            self.walker_group.load_or_create_model()
         for trial in range(self.trial):
             self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+        self._finish_with_model(configs, use_model)
+        return self.walker_group.to_config(self.walker_group.top1())
+
+    # ---- learned walk ---------------------------------------------------
+    def _q_schedule(self, configs, type_keys, use_model=False):
+        """Walk the space with one Q network per sub-space choosing directions
+        (flextensor/scheduler.py:444-540): warm up with random points, then per
+        trial take the best ``parallel`` points, step each of them once in every
+        sub-space, measure, store the transitions with reward
+        tanh(max(from - to, 0)), and train the walkers every trial/5 trials."""
+        self.walker_group.load_walker_model()
+        if use_model:
+            self.walker_group.load_or_create_model()
+        self._seed(configs, type_keys)
+        self._warm_up(min(self.warm_up_epoch, 10), self.warm_up_number, configs, type_keys,
+                      use_model=use_model)
+        best = self.walker_group.top1()
+        best_value = self.walker_group.top1_value()
+        retired_indices = []
+        value_early_stop = best_value
+        early_stop_count = 0
+        cur_lst = self.walker_group.topk(self.parallel, modify=True, with_value=True)
+        part = math.ceil(self.trial / 5)
+        for trial in range(self.trial):
+            from_lst, next_points, action_lst = self.walker_group.walk(cur_lst, trial)
+            results = self._cost(configs, next_points, use_model)
+            self._log("walk [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+            for indices, action, (from_indices, from_value), result in zip(next_points, action_lst,
+                                                                           from_lst, results):
+                gain = from_value - result if result < float("inf") else 0.0
+                if not use_model and from_value < float("inf"):
+                    gain = gain / from_value * 10.0      # kernels run for microseconds: scale to the start point
+                reward = float(np.tanh(max(gain, 0.0)))
+                self.walker_group.add_data(action[0], from_indices, action[1], indices, reward)
+                if result < float("inf"):
+                    self.walker_group.record(indices, result, random_reject=True)
+                else:
+                    self.walker_group.visit.add(str(indices))
+            if self.walker_group.top1_value() < best_value:
+                best_value = self.walker_group.top1_value()
+                best = self.walker_group.top1()
+            for indices, value in cur_lst:
+                if value < best_value:
+                    best, best_value = indices, value
+            self._log("No. %d | [%.6f] The best currently %.6f" % (trial, time.time(), best_value), best)
+            if value_early_stop < float("inf") and \
+                    math.fabs(best_value - value_early_stop) < 0.02 * value_early_stop:
+                early_stop_count += 1
+            else:
+                value_early_stop = best_value
+                early_stop_count = 0
+            if early_stop_count >= self.early_stop:
+                self._log("Early stop with value %f repeats %d times" % (value_early_stop, early_stop_count))
+                break
+            retired_indices.extend(cur_lst)
+            if not self.walker_group.has_more():
+                self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+                if not self.walker_group.has_more():
+                    self._log("No more points, end of scheduling")
+                    break
+            cur_lst = self.walker_group.topk(self.parallel, modify=True, with_value=True)
+            if (trial + 1) % part == 0:
+                self.walker_group.train_walkers()
+                if not use_model:
+                    # re-measure the leaders one after another
+                    for indices, value in retired_indices[-self.parallel:] + cur_lst:
+                        self.walker_group.record(indices, value, random_reject=False)
+                    indices_lst = self.walker_group.topk(self.parallel, modify=True)
+                    results = self._cost(configs, indices_lst, use_model=False)
+                    self._log("re-evaluate [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+                    for indices, result in zip(indices_lst, results):
+                        if result < float("inf"):
+                            self.walker_group.record(indices, result, random_reject=False)
+                    if indices_lst:
+                        best, best_value = {}, float("inf")
+                self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+                if self.walker_group.top1_value() < best_value:
+                    best_value = self.walker_group.top1_value()
+                    best = self.walker_group.top1()
+                cur_lst = self.walker_group.topk(self.parallel, modify=True, with_value=True)
+        # everything still held outside the heap goes back before the final pick
+        for indices, value in retired_indices + cur_lst:
+            if value < float("inf"):
+                self.walker_group.record(indices, value, random_reject=False)
+        if best and best_value < float("inf"):
+            self.walker_group.record(best, best_value, random_reject=False)
+        self._finish_with_model(configs, use_model)
+        self.walker_group.dump_data()
+        self.walker_group.clear_data()
         return self.walker_group.to_config(self.walker_group.top1())
 
     # ---- neighbourhood search -----------------------------------------
     def _searching_schedule(self, configs, type_keys, use_model=False):
+        if use_model:
+            self.walker_group.load_or_create_model()
         self._seed(configs, type_keys)
         self._warm_up(self.warm_up_epoch, self.warm_up_number, configs, type_keys,
                       use_model=use_model)
@@ -309,8 +426,7 @@ class Scheduler(object):
                 count_incessant_empty_trial += 1
             else:
                 count_incessant_empty_trial = 0
-            results = self.parallel_evaluate(configs, next_configs, number=self.number)
-            self.walker_group.add_perf_data(next_indices_lst, results)
+            results = self._cost(configs, next_indices_lst, use_model)
             self._log("tune [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
             rewards = [np.tanh(max(from_value - result, 0.0)) for result in results]
 
@@ -360,14 +476,20 @@ class Scheduler(object):
                 minimal = [{}, float("inf")]
                 indices_lst = self.walker_group.topk(self.re_evalutate_number, modify=True)
                 next_configs = [self.walker_group.to_config(indices) for indices in indices_lst]
-                results = self.parallel_evaluate(configs, next_configs, number=self.number)
-                self.walker_group.add_perf_data(indices_lst, results)
+                results = self._cost(configs, indices_lst, use_model)
                 self._log("re-evaluate [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
                 for indices, result in zip(indices_lst, results):
                     if result < float("inf"):
                         self.walker_group.record(indices, result, random_reject=False)
                 self.walker_group.clear_data()
             self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+        if use_model:
+            if minimal[1] < float("inf"):
+                self.walker_group.record(minimal[0], minimal[1], random_reject=False)
+            for retired in retired_indices:
+                self.walker_group.record(retired[0], retired[1], random_reject=False)
+            self._finish_with_model(configs, use_model)
+            return self.walker_group.to_config(self.walker_group.top1())
         if self.walker_group.top1_value() < minimal[1]:
             best = self.walker_group.top1()
         else:
@@ -438,12 +560,14 @@ class OpScheduler(Scheduler):
 
     def schedule(self, configs, method="searching", use_model=False, perf_path=None):
         wanted_types = ["fuse", "reorder", "spatial", "reduce", "unroll"]
-        if use_model:
-            raise RuntimeError("Currently no support for learned performance models")
+        if perf_path is not None:
+            self.walker_group.model_dir = perf_path
         if method == "searching":
             return self._searching_schedule(configs, wanted_types, use_model=use_model)
         elif method == "random":
             return self._random_schedule(configs, wanted_types, use_model=use_model)
+        elif method == "q":
+            return self._q_schedule(configs, wanted_types, use_model=use_model)
         else:
             raise RuntimeError("Currently no support for method %s" % method)
 
@@ -470,12 +594,14 @@ class GraphScheduler(Scheduler):
 
     def schedule(self, configs, method="searching", use_model=False, perf_path=None):
         types = ["inline", "merge", "special"]
-        if use_model:
-            raise RuntimeError("Currently no support for learned performance models")
+        if perf_path is not None:
+            self.walker_group.model_dir = perf_path
         if method == "searching":
             return self._searching_schedule(configs, types, use_model=use_model)
         elif method == "random":
             return self._random_schedule(configs, types, use_model=use_model)
+        elif method == "q":
+            return self._q_schedule(configs, types, use_model=use_model)
         else:
             raise RuntimeError("Currently no support for method %s" % method)
 
@@ -504,14 +630,18 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
 
     Keyword extras understood (flextensor/scheduler.py:990-1014): ``trials``
     (per-op trial counts), ``force_inline``, ``rpc_info`` (must not request a
-    remote session), ``use_model`` (must be false). Additional: ``evaluator``
+    remote session), ``use_model`` (rank candidates with the learned
+    performance model instead of the device; the model's best points are
+    measured at the end), ``perf_path`` (directory of the walker / performance
+    model files; nothing is written without it). Additional: ``evaluator``
     (a cost function used instead of the GPU, for host-only tests),
     ``warm_up`` = (epochs, points per epoch), ``verbose``.
+    ``method``: "searching", "random" or "q" (learned walkers).
     """
     task = TASK_TABLE[task_key]
     if task.target not in SUPPORTED_TARGETS:
         raise RuntimeError("Currently no support for target %s" % task.target)
-    if method not in ("searching", "random"):
+    if method not in ("searching", "random", "q"):
         raise RuntimeError("Currently no support for method %s" % method)
     ops, bufs = task.func(*task.args)
     op_lst, down_graph = flatten_graph(ops)
@@ -522,8 +652,8 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
         force_trials = kwargs["trials"]
     else:
         force_trials = [op_trial for _ in op_lst]
-    if kwargs.get("use_model"):
-        raise RuntimeError("Currently no support for learned performance models")
+    use_model = bool(kwargs.get("use_model", False))
+    perf_path = kwargs.get("perf_path")
     force_inline = bool(kwargs.get("force_inline", False))
     rpc_info = kwargs.get("rpc_info")
     if rpc_info is not None and getattr(rpc_info, "use_rpc", None):
@@ -563,7 +693,8 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
             if warm_up:
                 op_scheduler.warm_up_epoch, op_scheduler.warm_up_number = warm_up
             schedulers.append(op_scheduler)
-            op_config = op_scheduler.schedule(configs, method=method)
+            op_config = op_scheduler.schedule(configs, method=method, use_model=use_model,
+                                              perf_path=perf_path)
             configs.op_config_lst.append(op_config)
 
         if verbose:
@@ -580,7 +711,8 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
             graph_scheduler.warm_up_epoch = 2
             graph_scheduler.warm_up_number = min(20, max(len(graph_space), 1))
         schedulers.append(graph_scheduler)
-        graph_config = graph_scheduler.schedule(configs, method=method)
+        graph_config = graph_scheduler.schedule(configs, method=method, use_model=use_model,
+                                                perf_path=perf_path)
         configs = Config(configs.op_config_lst, graph_config)
     finally:
         for sch in schedulers:

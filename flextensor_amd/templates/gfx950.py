@@ -169,7 +169,8 @@ def _gemm_space(view):
     space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
-    space.add_subspace("xcd_remap", EnumSpace([[1, 0], [0, 0]] if i8 else [[1, 0], [0, 0], [1, 1], [0, 1], [1, 0, 1], [1, 0, 2]]),
+    space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
+                                            [[1, 0, 0], [0, 0, 0], [1, 1, 0], [0, 1, 0], [1, 0, 1], [1, 0, 2]]),
                        "reorder")
     return space
 
@@ -514,7 +515,7 @@ def default_config(op):
         cfg["reduce"] = [[1, view.KP // bk, bk]]
         cfg["unroll"] = [[2, 1]] if i8 else [[3, 1]]
         cfg["fuse"] = [[4]]
-        cfg["reorder"] = [[1, 0]]
+        cfg["reorder"] = [[1, 0, 0]]
     elif op.kind == "depthwise_conv2d_nchw":
         b, c, p, q = [x.extent for x in op.axis]
         th = 4 if p >= 4 else 1

@@ -514,12 +514,13 @@ def test_builtplan_rejects_mismatched_tensors():
     f.close()
 
 
-def test_schedule_on_device_small_gemm(oracle):
+@pytest.mark.parametrize("method", ["searching", "q"])
+def test_schedule_on_device_small_gemm(oracle, method):
     """End to end: search a few points on the GPU, replay the winner, check it."""
     np.random.seed(0)
     key = "gemm_gemm_(512, 256, 512)_rocm(0)"
     s, bufs, configs = schedule(key, op_trial=2, graph_trial=1, op_stop=2, parallel=8, number=5,
-                                timeout=20, warm_up=(1, 8), verbose=False)
+                                timeout=20, warm_up=(1, 8), verbose=False, method=method)
     a, b = seeded_inputs(bufs, 11)
     out = run_plan(key, configs, [a, b])
     assert rel(out, oracle.gemm_np(a, b)) <= TOL

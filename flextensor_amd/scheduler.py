@@ -635,7 +635,8 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
     measured at the end), ``perf_path`` (directory of the walker / performance
     model files; nothing is written without it). Additional: ``evaluator``
     (a cost function used instead of the GPU, for host-only tests),
-    ``warm_up`` = (epochs, points per epoch), ``verbose``.
+    ``warm_up`` = (epochs, points per epoch), ``verbose``, ``warm_start``
+    (default true: start from the shipped log's entry for this task, if any).
     ``method``: "searching", "random" or "q" (learned walkers).
     """
     task = TASK_TABLE[task_key]
@@ -672,6 +673,19 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
         configs = Config([], {"inline": [graph_space.subspaces["inline"].static_entities[0]]})
     else:
         configs = Config([], None)
+        # Operators are searched before the graph level, i.e. under the graph
+        # level's defaults. When the shipped log knows this task, its graph
+        # config (inline flags, special knobs) is the context instead, so that
+        # the shipped point keeps its measured cost when it seeds the search.
+        if kwargs.get("warm_start", True):
+            try:
+                from .tuned import lookup
+                shipped = lookup(task_key)
+                if shipped is not None and shipped.graph_config and \
+                        len(shipped.graph_config.get("special") or []) == len(task.special_space):
+                    configs = Config([], dict(shipped.graph_config))
+            except Exception:  # noqa: BLE001
+                pass
 
     schedulers = []
     try:

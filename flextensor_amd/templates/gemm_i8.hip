@@ -25,6 +25,10 @@
 //   XCD_REMAP   1: consecutive logical tiles stay on one XCD
 //   PAD         LDS row padding in bytes (multiple of 16); -1 selects
 //               unpadded rows whose 16-byte chunks are XOR-swizzled by row
+//   DTL         1: tiles travel global -> LDS directly (buffer loads with the
+//               lds modifier, 16 bytes per lane): no staging registers, no
+//               LDS store instructions; the row swizzle is applied on the
+//               global side, since a wavefront's 64 chunks land contiguously
 //   NT_STORE    1: non-temporal stores for C
 //   CVEC        1: the MFMA operands are swapped (the core computes the
 //               transposed tile), so a lane holds four consecutive columns of
@@ -55,6 +59,11 @@
 #define XCD_REMAP FT_XCD_REMAP
 #define PAD FT_PAD
 #define NT_STORE FT_NT_STORE
+#ifdef FT_DTL
+#define DTL FT_DTL
+#else
+#define DTL 0
+#endif
 #ifdef FT_CVEC
 #define CVEC FT_CVEC
 #else
@@ -119,6 +128,12 @@ typedef i32x4 acc_t;
 #define B_CHUNKS (BN * CHUNKS_ROW)
 #define EA ((A_CHUNKS + NT - 1) / NT)
 #define EB ((B_CHUNKS + NT - 1) / NT)
+#if DTL
+#if PAD > 0 || STAGES != 2 || A_CHUNKS % NT != 0 || B_CHUNKS % NT != 0
+#error "direct-to-LDS tiles need unpadded rows, two buffers and whole rounds of chunks"
+#endif
+typedef __attribute__((address_space(3))) void lds_void;
+#endif
 
 extern "C" __global__ __launch_bounds__(NT)
 void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ B,
@@ -154,13 +169,23 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     for (int e = 0; e < EA; ++e) {
         const int q = tid + e * NT;
         a_row[e] = q / CHUNKS_ROW;
+#if DTL
+        /* chunk q lands at byte 16*q of the tile = physical chunk q % CHUNKS_ROW
+         * of its row: fetch the logical chunk that belongs there */
+        a_col[e] = ((q % CHUNKS_ROW) ^ SWZ(a_row[e])) * 16;
+#else
         a_col[e] = (q % CHUNKS_ROW) * 16;
+#endif
     }
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
         const int q = tid + e * NT;
         b_row[e] = q / CHUNKS_ROW;
+#if DTL
+        b_col[e] = ((q % CHUNKS_ROW) ^ SWZ(b_row[e])) * 16;
+#else
         b_col[e] = (q % CHUNKS_ROW) * 16;
+#endif
     }
 
     /* raw buffer loads: an element that must read as zero (edge tile, idle
@@ -243,7 +268,103 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         }
     };
 
-#if FRAGPF
+#if DTL
+    {
+        const int wv = __builtin_amdgcn_readfirstlane(wave);
+        /* The load is written as an instruction, not through the builtin: the
+         * compiler makes every later LDS read wait for a direct-to-LDS load it
+         * knows of (it cannot tell the two buffers apart), which would undo the
+         * overlap. Completion is tracked by hand: vmcnt(0) and a barrier at
+         * the end of every iteration. */
+        auto descriptor = [](const signed char* base, unsigned bytes) {
+            const unsigned long long p = (unsigned long long)base;
+            i32x4 d;                         /* raw buffer: base, stride 0, size in bytes, untyped dwords */
+            d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+            d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(p >> 32) & 0xffffu));
+            d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+            d[3] = 0x00020000;
+            return d;
+        };
+        const i32x4 ra = descriptor(A, (unsigned)(M * K));
+        const i32x4 rb = descriptor(B, (unsigned)(N * K));
+        auto dma16 = [&](const i32x4& rsrc, const signed char* dst, unsigned vo, int so) {
+            const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory");
+        };
+        auto dma_tile = [&](int kt, int buf) {
+            const int k0 = kt * BK;
+#pragma unroll
+            for (int e = 0; e < EA; ++e) {
+                unsigned vo = a_voff[e];
+                if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+                dma16(ra, &As[buf][(e * NT + wv * 64) * 16], vo, k0);
+            }
+#pragma unroll
+            for (int e = 0; e < EB; ++e) {
+                unsigned vo = b_voff[e];
+                if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
+                dma16(rb, &Bs[buf][(e * NT + wv * 64) * 16], vo, k0);
+            }
+        };
+        dma_tile(0, 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);     /* vmcnt(0): this wavefront's chunks are in LDS */
+        __syncthreads();
+#if DTL == 2
+        /* with fragment prefetch: the LDS reads of step t+1 are issued before
+         * the MFMAs of step t, across the tile boundary as well */
+        const int arow = wm * REP_M * MFMA + li;
+        const int brow = wn * REP_N * MFMA + li;
+        auto load_frags = [&](int buf, int kk, i32x4 (&fa)[REP_M], i32x4 (&fb)[REP_N]) {
+            const signed char* as = &As[buf][arow * SROW];
+            const signed char* bs = &Bs[buf][brow * SROW];
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
+                fa[i] = *reinterpret_cast<const i32x4*>(as + i * MFMA * SROW + PCOL(arow + i * MFMA, kk + 16 * lg));
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+                fb[j] = *reinterpret_cast<const i32x4*>(bs + j * MFMA * SROW + PCOL(brow + j * MFMA, kk + 16 * lg));
+        };
+        i32x4 fa[REP_M], fb[REP_N];
+        load_frags(0, 0, fa, fb);
+        for (int kt = 0; kt < KT; ++kt) {
+            const int cur = kt & 1;
+            if (kt + 1 < KT) dma_tile(kt + 1, cur ^ 1);
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += MFMA_K) {
+                i32x4 na[REP_M], nb[REP_N];
+                if (kk + MFMA_K < BK) {
+                    load_frags(cur, kk + MFMA_K, na, nb);
+                } else {
+                    /* tile kt has been read by everybody, tile kt+1 has landed */
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
+                    __syncthreads();
+                    if (kt + 1 < KT) load_frags(cur ^ 1, 0, na, nb);
+                }
+#pragma unroll
+                for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+                    for (int j = 0; j < REP_N; ++j)
+                        acc[i][j] = MFMA_OP(fa[i], fb[j], acc[i][j]);
+                if (kk + MFMA_K < BK || kt + 1 < KT) {
+#pragma unroll
+                    for (int i = 0; i < REP_M; ++i) fa[i] = na[i];
+#pragma unroll
+                    for (int j = 0; j < REP_N; ++j) fb[j] = nb[j];
+                }
+            }
+        }
+#else
+        for (int kt = 0; kt < KT; ++kt) {
+            const int cur = kt & 1;
+            if (kt + 1 < KT) dma_tile(kt + 1, cur ^ 1);   /* lands while tile kt is multiplied */
+            compute(cur);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        }
+#endif
+    }
+#elif FRAGPF
     {
         const int arow = wm * REP_M * MFMA + li;
         const int brow = wn * REP_N * MFMA + li;

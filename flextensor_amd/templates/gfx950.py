@@ -166,7 +166,7 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
     space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
@@ -213,7 +213,9 @@ SPECIAL_DEFAULTS = {
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
 # depth 5 = two stages with the fragment-prefetch pipeline (int8 GEMM)
-PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1)}
+# depth -> (LDS buffers, global prefetch distance); int8 only: 5 = MFMA fragment prefetch,
+# 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch
+PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7: (2, 1)}
 
 
 def special_knobs(kind):
@@ -252,7 +254,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE or (depth == 5 and view.dtype != "int8"):
+    if depth not in PIPELINE or (depth >= 5 and view.dtype != "int8"):
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
@@ -299,7 +301,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
             raise InvalidConfig("int8 LDS padding must be a multiple of 16 bytes")
         if view.M * view.K >= 2 ** 31 or view.N * view.K >= 2 ** 31:
             raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
-        if (ceil_div(bm * bk // 16, nt) + ceil_div(bn * bk // 16, nt)) * 4 * pd > 160:
+        if depth >= 6:
+            if pad > 0 or (bm * bk // 16) % nt or (bn * bk // 16) % nt:
+                raise InvalidConfig("direct-to-LDS tiles need unpadded rows and whole rounds of 16-byte chunks")
+        elif (ceil_div(bm * bk // 16, nt) + ceil_div(bn * bk // 16, nt)) * 4 * pd > 160:
             raise InvalidConfig("global->LDS staging needs too many registers")
         lds = stages * (bm + bn) * (bk + max(pad, 0))
         if lds > LDS_BYTES:
@@ -309,6 +314,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         if store_mode & 2 and view.N % 4 != 0:
             raise InvalidConfig("128-bit C stores need N to be a multiple of 4")
         D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0, NT_STORE=store_mode & 1)
+        if depth >= 6:
+            D.update(DTL=depth - 5)
         if store_mode & 2:
             D.update(CVEC=1)
         grid = (gm * gn, 1, 1)

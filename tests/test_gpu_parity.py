@@ -268,6 +268,13 @@ def test_gemm_transpose_b_vs_oracle(oracle):
     (200, 320, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, st=5)),       # same, ragged, one k-step per tile
     (256, 64, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=64, st=5)),        # same, a single tile
     (256, 768, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=4)),      # prefetch 3 tiles
+    (512, 512, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=6)),      # tiles straight into LDS
+    (200, 336, 136, dict(wm=2, rm=2, wn=1, rn=4, mf=16, bk=64, st=6)),       # same, ragged M, N and K tail
+    (256, 64, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=64, st=6)),        # same, a single tile
+    (512, 512, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, st=7)),      # straight into LDS + fragment prefetch
+    (200, 336, 136, dict(wm=2, rm=2, wn=1, rn=4, mf=16, bk=64, st=7)),       # same, ragged, one step per tile
+    (256, 64, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=64, st=7)),        # same, a single tile
+    (512, 1024, 512, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=256, st=7)),     # same, 16 wavefronts, four steps per tile
 ])
 def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
     _gemm_int8_case(oracle, M, K, N, kn, None)
@@ -292,9 +299,9 @@ def _gemm_int8_case(oracle, M, K, N, kn, store):
     a, b = seeded_inputs(bufs, seed=K)
     assert a.min() == -128 and a.max() == 127
     g = None
-    if store is not None:
+    if store is not None or kn.get("st") in (6, 7):       # direct-to-LDS tiles need the swizzled (unpadded) layout
         g = {k: [] for k in KEYS}
-        g["inline"], g["special"] = [[0]], [[-1, 0], [store]]
+        g["inline"], g["special"] = [[0]], [[-1, 0], [store or 0]]
     out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], g), [a, b])
     assert np.array_equal(out, oracle.gemm_i8_c(a, b))
     assert np.array_equal(out, oracle.gemm_i8_np(a, b))

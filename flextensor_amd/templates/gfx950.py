@@ -166,7 +166,7 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7] if i8 else [1, 2, 3, 4], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7] if i8 else [1, 2, 3, 4, 5], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
     space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
@@ -213,7 +213,8 @@ SPECIAL_DEFAULTS = {
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
 # depth 5 = two stages with the fragment-prefetch pipeline (int8 GEMM)
-# depth -> (LDS buffers, global prefetch distance); int8 only: 5 = MFMA fragment prefetch,
+# depth -> (LDS buffers, global prefetch distance); 5 = int8: MFMA fragment prefetch, fp32: tiles
+# loaded straight into LDS; int8 only:
 # 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch
 PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7: (2, 1)}
 
@@ -254,7 +255,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE or (depth >= 5 and view.dtype != "int8"):
+    if depth not in PIPELINE or (depth >= 6 and view.dtype != "int8"):
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     group_m = int((config.get("fuse") or [[4]])[0][0])
@@ -338,6 +339,18 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         bv = av
     else:
         bv = 1
+    dtl = depth == 5          # fp32: tiles loaded straight into LDS
+    if dtl:
+        if view.mode != 2:
+            bv = 1            # B goes one float per lane
+        if apad < 0 and (bk & (bk - 1)) != 0:
+            apad = 0          # rows land contiguously: unpadded when the swizzle is not available
+        if waves_k != 1 or av != 4 or apad > 0 or (bm * bk // 4) % 64:
+            raise InvalidConfig("direct-to-LDS tiles need 16-byte A chunks in whole wavefronts and unpadded A rows")
+        if view.mode == 2 and (bv != 4 or (bn * bk // 4) % 64):
+            raise InvalidConfig("direct-to-LDS tiles need 16-byte B chunks in whole wavefronts")
+        if view.mode != 2 and bn % 64:
+            raise InvalidConfig("direct-to-LDS tiles need BN to be a multiple of 64")
     if apad < 0 and (bk & (bk - 1)) != 0:
         apad = 4              # the chunk swizzle needs a power-of-two row
     sa = bk + max(apad, 0)
@@ -353,11 +366,13 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     # staging registers for the global->LDS copy must stay reasonable
     ea = ceil_div(bm * bk // av, nt)
     eb = ceil_div((bn * bk) // bv, nt)
-    if (ea * av + eb * bv) * pd > 160:
+    if not dtl and (ea * av + eb * bv) * pd > 160:
         raise InvalidConfig("global->LDS staging needs too many registers")
     if max(view.M * view.K, view.K * view.N, view.M * view.N) * view.groups * 4 >= 2 ** 31:
         raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
     D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
+    if dtl:
+        D.update(DTL=1)
     specs = []
     if view.mode == 1:
         conv = dict(view.conv)

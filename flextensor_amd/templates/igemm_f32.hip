@@ -30,6 +30,13 @@
 //                   WAVES_M*WAVES_N wavefronts each multiply their own K slice
 //                   through their own LDS tiles; the partial tiles are summed
 //                   through LDS at the end (no atomics, no zero fill)
+//   DTL             1: tiles travel global -> LDS directly (buffer loads with
+//                   the lds modifier): no staging registers and no LDS store
+//                   instructions. A (and B^T) in 16-byte chunks, 64 per
+//                   wavefront landing contiguously, so rows are unpadded and
+//                   the swizzle is applied on the global side; B one float
+//                   per lane, 64 consecutive columns of one k row per
+//                   instruction (BN % 64 == 0), rows still padded
 //   SK_PER          > 0: balanced K streaming. The work is cut into units of
 //                   one LDS tile step (output tile, k-tile); every workgroup
 //                   takes SK_PER consecutive units, so a workgroup may
@@ -74,6 +81,11 @@
 #define BPAD FT_BPAD
 #define AV FT_AV
 #define BV FT_BV
+#ifdef FT_DTL
+#define DTL FT_DTL
+#else
+#define DTL 0
+#endif
 #ifdef FT_SK_PER
 #define SK_PER FT_SK_PER
 #else
@@ -157,6 +169,22 @@ typedef f32x4 acc_t;
 #define B_CHUNKS (BK * B_CHUNKS_ROW)
 #endif
 #define EB ((B_CHUNKS + NT - 1) / NT)
+#if DTL
+#if WAVES_K != 1 || STAGES != 2 || PD != 1 || AV != 4 || APAD > 0 || A_CHUNKS % 64 != 0 || B_CHUNKS % 64 != 0
+#error "direct-to-LDS tiles: two buffers, 16-byte A chunks, unpadded A rows, whole wavefronts of chunks"
+#endif
+#if MODE == 2
+#if BV != 4
+#error "direct-to-LDS tiles: B^T needs 16-byte chunks"
+#endif
+#else
+#if BV != 1 || BN % 64 != 0
+#error "direct-to-LDS tiles: B goes one float per lane, 64 columns of a row per instruction"
+#endif
+#endif
+typedef __attribute__((address_space(3))) void lds_void;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+#endif
 
 #if AV == 4
 typedef f32x4 avec_t;
@@ -269,14 +297,24 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     for (int e = 0; e < EA; ++e) {
         const int q = tid + e * NT;
         a_row[e] = q / A_CHUNKS_ROW;
+#if DTL
+        /* chunk q lands at float 4*q of the tile, i.e. at physical chunk
+         * q % A_CHUNKS_ROW of its row: fetch the logical chunk that belongs there */
+        a_col[e] = ACOL(a_row[e], (q % A_CHUNKS_ROW) * AV);
+#else
         a_col[e] = (q % A_CHUNKS_ROW) * AV;
+#endif
     }
     int b_row[EB], b_col[EB];
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
         const int q = tid + e * NT;
         b_row[e] = q / B_CHUNKS_ROW;
+#if DTL && MODE == 2
+        b_col[e] = ACOL(b_row[e], (q % B_CHUNKS_ROW) * BV);
+#else
         b_col[e] = (q % B_CHUNKS_ROW) * BV;
+#endif
     }
     /* ---- workgroup -> (group, split, tile_m, tile_n) and K range -------- */
     /* tile index inside one group -> first row / column of the tile */
@@ -574,14 +612,91 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         }
     };
 
+#if DTL
+    /* The loads are written as instructions, not through the builtin: the
+     * compiler makes every later LDS read wait for a direct-to-LDS load it
+     * knows of (it cannot tell the two buffers apart), which would undo the
+     * overlap. Completion is tracked by hand: vmcnt(0) before the barrier
+     * that ends an iteration. */
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    auto descriptor = [](const float* base, unsigned bytes) {
+        const unsigned long long p = (unsigned long long)base;
+        i32x4 d;                             /* raw buffer: base, stride 0, bytes, untyped dwords */
+        d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+        d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(p >> 32) & 0xffffu));
+        d[2] = (int)bytes;
+        d[3] = 0x00020000;
+        return d;
+    };
+    const i32x4 desc_a = descriptor(A, (unsigned)A_BYTES);
+    const i32x4 desc_b = descriptor(B, (unsigned)B_BYTES);
+    auto dma16 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
+        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory");
+    };
+    auto dma4 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
+        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory");
+    };
+    auto dma_tile = [&](int kt, int buf) {
+        const int k0 = kbase + kt * BK;
+#pragma unroll
+        for (int e = 0; e < EA; ++e) {
+            unsigned vo = a_voff[e];
+            if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+            if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))     /* whole wavefronts only */
+                dma16(desc_a, &As[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
+        }
+#pragma unroll
+        for (int e = 0; e < EB; ++e) {
+            if (!((B_CHUNKS % NT == 0) || (e * NT + wv * 64 < B_CHUNKS))) continue;
+#if MODE == 2
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
+            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
+#else
+            /* the wavefront's 64 lanes are 64 consecutive columns of one k row */
+            const int q0 = e * NT + wv * 64;
+            const float* dst = &Bs[buf][(q0 / BN) * SB + (q0 % BN)];
+#if MODE == 0
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma4(desc_b, dst, vo, k0 * (N * 4));
+#elif KHOIST
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma4(desc_b, dst, vo, (k0 / (CR * CS)) * (CH * CW * 4));
+#else
+            const int k = k0 + b_row[e];
+            const int c = k / (CR * CS);
+            const int rs = k % (CR * CS);
+            const int ih = px_h[e] + (rs / CS) * CDIL;
+            const int iw = px_w[e] + (rs % CS) * CDIL;
+            bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+            if (KP != K) ok = ok && (k < K);
+            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
+            dma4(desc_b, dst, vo, 0);
+#endif
+#endif
+        }
+    };
+#endif
+
     /* ---- main loop ------------------------------------------------------ */
     /* Tile t travels global -> register set t % PD -> LDS buffer -> MFMA.
      * While tile kt is multiplied, tiles kt+1 .. kt+PD are in registers or in
      * flight; tile kt+1 is written to LDS right after the MFMAs of tile kt. */
+#if DTL
+    dma_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);      /* vmcnt(0): this wavefront's part of tile 0 is in LDS */
+#else
 #pragma unroll
     for (int p = 0; p < PD; ++p)
         if (p < nk) load_global(p, p);
     store_lds(0, 0);
+#endif
 #if SK_PER > 0
     /* The arrival for the slot written at the end of the previous segment is
      * counted here: the wait for this tile's first loads has covered the slot
@@ -596,6 +711,15 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         arrive_tile = -1;
     }
 #endif
+#if DTL
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) dma_tile(kt + 1, cur ^ 1);      /* lands while tile kt is multiplied */
+        compute(cur);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+    }
+#else
     for (int kt0 = 0; kt0 < nk; kt0 += PD) {
 #pragma unroll
         for (int u = 0; u < PD; ++u) {
@@ -613,6 +737,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             }
         }
     }
+#endif
 
 #if WAVES_K > 1
     /* ---- sum the k-groups' partial tiles through LDS --------------------- */

@@ -244,6 +244,67 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     func.close()
 
 
+@pytest.mark.parametrize("M,K,N,kn,pad", [
+    (256, 256, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, -1]),            # swizzled A rows
+    (256, 512, 256, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=64, st=5), [-1, 4]),
+    (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=5), [0, 8]),               # ragged M, N; padded K
+    (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=5, ks=1), [-1, -1]),      # with K streaming
+    (96, 144, 128, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=72, st=5), [0, 0]),               # partial last round of chunks
+])
+def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
+    """Pipeline depth 5: tiles travel global -> LDS without staging registers."""
+    register(gemm, "gemm", "gemm", (M, K, N), "rocm", 0)
+    key = key_of("gemm", "gemm", (M, K, N))
+    ops, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=M + N)
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[0]], [pad]
+    s, _ = schedule_with_config(key, Config([gcfg(M, N, kp, **kn)], g))
+    assert s.specs[-1].defines["DTL"] == 1
+    out = run_plan(key, Config([gcfg(M, N, kp, **kn)], g), [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+
+
+def test_gemm_transpose_b_direct_to_lds(oracle):
+    def wrap(M, K, N):
+        A = placeholder((M, K), name="A")
+        B = placeholder((N, K), name="B")
+        C = op_gemm(A, B, transposeB=True)
+        return [C.op], [A, B, C]
+    register(wrap, "gemm", "gemm_nt", (160, 96, 224), "rocm", 0)
+    key = key_of("gemm", "gemm_nt", (160, 96, 224))
+    TASK_TABLE[key].set_specific_space("lds_pad", "enum", [[-1, -1]])
+    _, bufs = wrap(160, 96, 224)
+    a, b = seeded_inputs(bufs, seed=9)
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[0]], [[-1, -1]]
+    out = run_plan(key, Config([gcfg(160, 224, 96, 2, 1, 2, 1, 32, 32, st=5)], g), [a, b])
+    assert rel(out, oracle.gemm_f32_c(a, b, transB=True)) <= TOL
+
+
+@pytest.mark.parametrize("args,kn,pad", [
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=16, st=5), [-1, 8]),
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=5), [0, 0]),     # groups, hoisted gather
+    ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=2, wn=4, rn=1, mf=16, bk=16, st=5), [-1, 4]),     # stride 2, K tail
+    ((3, 8, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=16, st=5, ks=1), [-1, 4]),   # dilation, K streaming
+    ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, 8]),      # 1x1, N=392
+])
+def test_conv2d_direct_to_lds(oracle, args, kn, pad):
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    key = key_of("conv2d", "t", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
+    M, N, K = ko // g, nb * ref.shape[2] * ref.shape[3], (c // g) * ks * ks
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    cfg = gcfg(M, N, kp, **kn)
+    for inline in ([1, 0], [0, 0]):
+        out = run_plan(key, conv_cfgs(cfg, inline, [pad]), [x, w])
+        assert rel(out, ref) <= TOL, inline
+
+
 def test_gemm_transpose_b_vs_oracle(oracle):
     def wrap(M, K, N):
         A = placeholder((M, K), name="A")

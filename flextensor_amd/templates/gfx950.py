@@ -141,7 +141,7 @@ class GemmView(object):
         self.KP = self.KP_options[-1]
 
 
-F32_BK = (8, 16, 32, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
+F32_BK = (8, 16, 32, 48, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
 I8_BK = (64, 128, 256)
 
 
@@ -345,12 +345,12 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
             bv = 1            # B goes one float per lane
         if apad < 0 and (bk & (bk - 1)) != 0:
             apad = 0          # rows land contiguously: unpadded when the swizzle is not available
-        if waves_k != 1 or av != 4 or apad > 0 or (bm * bk // 4) % 64:
+        if av != 4 or apad > 0 or (bm * bk // 4) % 64:
             raise InvalidConfig("direct-to-LDS tiles need 16-byte A chunks in whole wavefronts and unpadded A rows")
         if view.mode == 2 and (bv != 4 or (bn * bk // 4) % 64):
             raise InvalidConfig("direct-to-LDS tiles need 16-byte B chunks in whole wavefronts")
-        if view.mode != 2 and bn % 64:
-            raise InvalidConfig("direct-to-LDS tiles need BN to be a multiple of 64")
+        if view.mode != 2 and bn % 64 and not (64 % bn == 0 and bpad == 0 and (bn * bk) % 64 == 0):
+            raise InvalidConfig("direct-to-LDS tiles need BN % 64 == 0, or BN dividing 64 with unpadded B rows")
     if apad < 0 and (bk & (bk - 1)) != 0:
         apad = 4              # the chunk swizzle needs a power-of-two row
     sa = bk + max(apad, 0)

@@ -35,8 +35,9 @@
 //                   instructions. A (and B^T) in 16-byte chunks, 64 per
 //                   wavefront landing contiguously, so rows are unpadded and
 //                   the swizzle is applied on the global side; B one float
-//                   per lane, 64 consecutive columns of one k row per
-//                   instruction (BN % 64 == 0), rows still padded
+//                   per lane: 64 consecutive columns of one k row per
+//                   instruction (BN % 64 == 0, rows may be padded) or whole
+//                   unpadded rows (BN < 64)
 //   SK_PER          > 0: balanced K streaming. The work is cut into units of
 //                   one LDS tile step (output tile, k-tile); every workgroup
 //                   takes SK_PER consecutive units, so a workgroup may
@@ -170,7 +171,7 @@ typedef f32x4 acc_t;
 #endif
 #define EB ((B_CHUNKS + NT - 1) / NT)
 #if DTL
-#if WAVES_K != 1 || STAGES != 2 || PD != 1 || AV != 4 || APAD > 0 || A_CHUNKS % 64 != 0 || B_CHUNKS % 64 != 0
+#if STAGES != 2 || PD != 1 || AV != 4 || APAD > 0 || A_CHUNKS % 64 != 0 || B_CHUNKS % 64 != 0
 #error "direct-to-LDS tiles: two buffers, 16-byte A chunks, unpadded A rows, whole wavefronts of chunks"
 #endif
 #if MODE == 2
@@ -178,8 +179,8 @@ typedef f32x4 acc_t;
 #error "direct-to-LDS tiles: B^T needs 16-byte chunks"
 #endif
 #else
-#if BV != 1 || BN % 64 != 0
-#error "direct-to-LDS tiles: B goes one float per lane, 64 columns of a row per instruction"
+#if BV != 1 || !(BN % 64 == 0 || (64 % BN == 0 && BPAD == 0))
+#error "direct-to-LDS tiles: B goes one float per lane; a wavefront covers part of one row, or whole unpadded rows"
 #endif
 #endif
 typedef __attribute__((address_space(3))) void lds_void;

@@ -289,6 +289,8 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=2, wn=4, rn=1, mf=16, bk=16, st=5), [-1, 4]),     # stride 2, K tail
     ((3, 8, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=16, st=5, ks=1), [-1, 4]),   # dilation, K streaming
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, 8]),      # 1x1, N=392
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=16, sk=4, wk=1, st=5), [0, 0]),   # BN=16, 4 k-groups
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=72, sk=2, wk=1, st=5), [0, 0]),   # BN=32, whole windows
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)

@@ -16,6 +16,12 @@
 // lanes through DPP wavefront shifts instead of two more global loads; each
 // wavefront then uses a multiple of TILES_W lanes so that neighbours along W
 // are always in the same wavefront).
+// LDSP > 0 selects the plane-staged variant instead: a workgroup streams LDSP
+// whole planes into LDS with 128-bit loads in pure copy order (every input
+// element is fetched once, no halo re-reads), computes from LDS, where a zero
+// border stands for the padding, and writes the outputs in the same order.
+// It needs a same-size 3x3 / stride 1 / dilation 1 / padding 1 layer with
+// FACT == 1 and rows that are multiples of four floats.
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
 // STR, PAD, DIL, FACT, CP x CQ output.
 
@@ -26,6 +32,16 @@
 #define TW FT_TW
 #define NT_STORE FT_NT_STORE
 #define SHFL FT_SHFL
+#ifdef FT_NT_LOAD
+#define NT_LOAD FT_NT_LOAD
+#else
+#define NT_LOAD 0
+#endif
+#ifdef FT_LDSP
+#define LDSP FT_LDSP
+#else
+#define LDSP 0
+#endif
 #define CB FT_CB
 #define CC FT_CC
 #define CH FT_CH
@@ -69,6 +85,86 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define LPW 64
 #endif
 
+#if LDSP > 0
+#if !(STR == 1 && DIL == 1 && CR == 3 && CS == 3 && PAD == 1 && CP == CH && CQ == CW && CW % 4 == 0 && FACT == 1)
+#error "the plane-staged variant needs a same-size 3x3 stride-1 pad-1 layer, FACT 1, CW % 4 == 0"
+#endif
+#define RS (CW + 8)                  /* LDS row: 4 zero floats, CW data, 4 zero floats */
+#define PS ((CH + 2) * RS)           /* plane: zero row, CH rows, zero row */
+#define Q4 (CW / 4)                  /* 128-bit chunks per row */
+#define PLANE4 (CH * Q4)             /* ... per plane */
+#define BORDER4 (2 * (RS / 4) + 2 * CH)   /* border chunks per plane: two rows + two per data row */
+
+extern "C" __global__ __launch_bounds__(NT)
+void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
+                   float* __restrict__ O)
+{
+    __shared__ __attribute__((aligned(16))) float sx[LDSP * PS];
+    __shared__ __attribute__((aligned(16))) float sw[LDSP * 12];     /* 3 taps + 1 pad per kernel row */
+    const int tid = threadIdx.x;
+    const int p0 = blockIdx.x * LDSP;
+    const f32x4 zero = (f32x4)(0.0f);
+    /* ---- borders (the padding) ---------------------------------------- */
+    for (int i = tid; i < LDSP * BORDER4; i += NT) {
+        const int pl = i / BORDER4;
+        const int q = i % BORDER4;
+        int off;
+        if (q < RS / 4) off = q * 4;                                   /* top row */
+        else if (q < 2 * (RS / 4)) off = (CH + 1) * RS + (q - RS / 4) * 4;   /* bottom row */
+        else {
+            const int k = q - 2 * (RS / 4);                            /* left / right of a data row */
+            off = (k / 2 + 1) * RS + ((k & 1) ? (CW + 4) : 0);
+        }
+        *reinterpret_cast<f32x4*>(&sx[pl * PS + off]) = zero;
+    }
+    /* ---- weights: [plane][r][s] -> [plane][r][4] ------------------------ */
+    for (int i = tid; i < LDSP * 9; i += NT) {
+        const int pl = i / 9, k = i % 9;
+        const int plane = p0 + pl;
+        sw[pl * 12 + (k / 3) * 4 + (k % 3)] = (plane < PLANES) ? Wt[(size_t)(plane % (CC * FACT)) * 9 + k] : 0.0f;   /* kernels repeat per batch entry */
+    }
+    /* ---- planes, in copy order ------------------------------------------ */
+    const f32x4* X4 = reinterpret_cast<const f32x4*>(X);
+    for (int i = tid; i < LDSP * PLANE4; i += NT) {
+        const int pl = i / PLANE4;
+        const int rem = i % PLANE4;
+        const int plane = p0 + pl;
+        f32x4 v = zero;
+        if (plane < PLANES) v = NT_LOAD ? __builtin_nontemporal_load(&X4[(size_t)plane * PLANE4 + rem])
+                                        : X4[(size_t)plane * PLANE4 + rem];
+        *reinterpret_cast<f32x4*>(&sx[pl * PS + (rem / Q4 + 1) * RS + 4 + (rem % Q4) * 4]) = v;
+    }
+    __syncthreads();
+    /* ---- four outputs per item, same order ------------------------------ */
+    f32x4* O4 = reinterpret_cast<f32x4*>(O);
+    for (int i = tid; i < LDSP * PLANE4; i += NT) {
+        const int pl = i / PLANE4;
+        const int rem = i % PLANE4;
+        const int plane = p0 + pl;
+        if (plane >= PLANES) break;
+        const float* base = &sx[pl * PS + (rem / Q4) * RS + 4 + (rem % Q4) * 4];   /* input row of tap r = 0 */
+        f32x4 acc = zero;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const f32x4 w = *reinterpret_cast<const f32x4*>(&sw[pl * 12 + r * 4]);
+            const f32x4 m = *reinterpret_cast<const f32x4*>(base + r * RS);
+            const float l = base[r * RS - 1];
+            const float g = base[r * RS + 4];
+            const float in[6] = {l, m[0], m[1], m[2], m[3], g};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+                    acc[j] += in[j + t] * w[t];
+        }
+#if NT_STORE
+        __builtin_nontemporal_store(acc, &O4[(size_t)plane * PLANE4 + rem]);
+#else
+        O4[(size_t)plane * PLANE4 + rem] = acc;
+#endif
+    }
+}
+#else
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                    float* __restrict__ O)
@@ -121,7 +217,8 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #if SHFL
         {
             f32x4 v = (f32x4)(0.0f);
-            if (row_ok) v = *reinterpret_cast<const f32x4*>(xr + ow0);
+            if (row_ok) v = NT_LOAD ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + ow0))
+                                   : *reinterpret_cast<const f32x4*>(xr + ow0);
             /* column ow0-1 is the last column of the lane below, column ow0+4
              * the first column of the lane above; image borders read zero */
             const float v0 = v[0], v3 = v[3];
@@ -134,7 +231,8 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #elif VEC_IN
         {
             f32x4 v = (f32x4)(0.0f);
-            if (row_ok) v = *reinterpret_cast<const f32x4*>(xr + ow0);
+            if (row_ok) v = NT_LOAD ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + ow0))
+                                   : *reinterpret_cast<const f32x4*>(xr + ow0);
 #pragma unroll
             for (int j = 0; j < IW_T; ++j) {
                 if (j >= PAD && j < PAD + 4) {
@@ -189,3 +287,4 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #endif
     }
 }
+#endif

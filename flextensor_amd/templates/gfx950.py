@@ -209,6 +209,7 @@ SPECIAL_DEFAULTS = {
     "lds_pad": [4, -1],
     "nt_store": [0],
     "halo_shfl": [0],
+    "lds_planes": [0],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -227,7 +228,7 @@ def special_knobs(kind):
     if kind == "gemm_int8":
         return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
-        return {"nt_store": [[0], [1]], "halo_shfl": [[0], [1]]}
+        return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]]}
     return {}
 
 
@@ -443,6 +444,21 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         raise InvalidConfig("lane patch needs too many registers")
     nt = waves * 64
     items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
+    ldsp = int(_special(special, "lds_planes")[0])
+    nt_mode = int(_special(special, "nt_store")[0])     # bit 0: non-temporal stores, bit 1: non-temporal loads
+    if ldsp:
+        # plane-staged variant: whole planes through LDS in copy order; the lane patch knobs do not apply
+        st, dl = a["stride"][0], a["dilation"][0]
+        if not (st == 1 and dl == 1 and r_ext == 3 and s_ext == 3 and pad == 1 and p == h and q == w
+                and w % 4 == 0 and a["factor"] == 1):
+            raise InvalidConfig("plane staging needs a same-size 3x3 stride-1 pad-1 layer with rows of whole vectors")
+        if ldsp < 0 or (ldsp * (h + 2) * (w + 8) + ldsp * 12) * 4 > LDS_BYTES:
+            raise InvalidConfig("staged planes do not fit the LDS")
+        D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=0, LDSP=ldsp,
+                 CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=1, PAD=1, DIL=1, FACT=1, CP=p, CQ=q)
+        return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(b * cout, ldsp), 1, 1),
+                           (nt, 1, 1),
+                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
     shfl = int(_special(special, "halo_shfl")[0])
     tiles_w = ceil_div(q, tw)
     if shfl:
@@ -453,7 +469,7 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         grid_x = ceil_div(ceil_div(items, lanes), waves)
     else:
         grid_x = ceil_div(items, nt)
-    D = dict(NT=nt, TH=th, TW=tw, NT_STORE=int(_special(special, "nt_store")[0]), SHFL=shfl,
+    D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=shfl,
              CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=a["stride"][0], PAD=pad,
              DIL=a["dilation"][0], FACT=a["factor"], CP=p, CQ=q)
     del ih_t

@@ -440,13 +440,44 @@ def test_depthwise_shuffled_halo_vs_oracle(oracle, args, th, waves):
     x, w = seeded_inputs(bufs, seed=sum(args))
     ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
     b_, co, p, q = ref.shape
-    for nt_store in (0, 1):
+    for nt_store in (0, 1, 3):                    # bit 0: non-temporal stores, bit 1: non-temporal loads
         out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, 4, waves), special=[[nt_store], [1]]), [x, w])
         assert rel(out, ref) <= TOL, nt_store
     # borders: a constant image must give border sums with missing taps
     ones = np.ones_like(x)
     out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, 4, waves), special=[[0], [1]]), [ones, w])
     assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
+
+
+@pytest.mark.parametrize("args,planes,waves", [
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 4, 4),
+    ((1, 5, 8, 12, 1, 3, 1, 1, 1), 2, 1),         # 5 planes, 2 per workgroup: the last workgroup is half empty
+    ((3, 7, 16, 64, 1, 3, 1, 1, 1), 1, 2),
+    ((2, 3, 7, 4, 1, 3, 1, 1, 1), 8, 1),          # one vector per row, more slots than planes
+])
+def test_depthwise_plane_staged_vs_oracle(oracle, args, planes, waves):
+    """Whole planes staged through LDS in copy order; a zero border is the padding."""
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
+    b_, co, p, q = ref.shape
+    for nt_store in (0, 1, 2):
+        cfgs = conv_cfgs(dcfg(b_, co, p, q, 1, 4, waves), special=[[nt_store], [0], [planes]])
+        s, _ = schedule_with_config(key, cfgs)
+        assert s.specs[-1].defines["LDSP"] == planes
+        out = run_plan(key, cfgs, [x, w])
+        assert rel(out, ref) <= TOL, nt_store
+    ones = np.ones_like(x)
+    out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, 1, 4, waves), special=[[0], [0], [planes]]), [ones, w])
+    assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
+    # a layer it does not fit is refused, not mis-computed
+    bad = (1, 4, 9, 20, 2, 3, 1, 1, 1)            # factor 2
+    register(depthwise_conv2d, "conv2d", "depthwise", bad, "rocm", 0)
+    with pytest.raises(Exception):
+        schedule_with_config(key_of("conv2d", "depthwise", bad),
+                             conv_cfgs(dcfg(1, 8, 9, 20, 1, 4, 1), special=[[0], [0], [2]]))
 
 
 def test_default_schedule_kernels_vs_oracle(oracle):

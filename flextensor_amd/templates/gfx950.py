@@ -329,6 +329,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
     if bk % kblk != 0:
         raise InvalidConfig("BK must be a multiple of %d for this MFMA shape" % kblk)
     apad, bpad = [int(x) for x in _special(special, "lds_pad")[:2]]
+    bpad_auto = bpad < 0
     if bpad < 0:
         bpad = 4 if mfm == 16 else 8
     if apad < -1 or (apad >= 0 and apad % 4 != 0) or bpad % 4 != 0:
@@ -342,7 +343,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         bv = 1
     dtl = depth == 5          # fp32: tiles loaded straight into LDS
     if dtl:
-        if view.mode != 2:
+        if view.mode == 0 and view.N % 4 == 0 and bn % 64 == 0 and (bpad_auto or bpad == 0):
+            bv, bpad = 4, 0   # B in 16-byte chunks too: unpadded rows, columns swizzled by k
+        elif view.mode != 2:
             bv = 1            # B goes one float per lane
         if apad < 0 and (bk & (bk - 1)) != 0:
             apad = 0          # rows land contiguously: unpadded when the swizzle is not available

@@ -179,7 +179,21 @@ typedef f32x4 acc_t;
 #error "direct-to-LDS tiles: B^T needs 16-byte chunks"
 #endif
 #else
-#if BV != 1 || !(BN % 64 == 0 || (64 % BN == 0 && BPAD == 0))
+#if MODE == 0 && BV == 4
+/* B in 16-byte chunks as well: rows land unpadded, so the four k rows that the
+ * lane groups of an MFMA read together would hit the same banks; instead the
+ * chunks of row k are XOR-ed (on the global side) by a function of k that moves
+ * each lane group to its own banks. */
+#if BPAD != 0 || BN % 64 != 0
+#error "direct-to-LDS B in 16-byte chunks needs unpadded rows of a multiple of 64 floats"
+#endif
+#define BSWZ 1
+#if MFMA == 16
+#define BSWK(k) ((((k) >> 2) & 3) << 2)     /* chunk XOR of row k: 16 floats per lane group */
+#else
+#define BSWK(k) ((((k) >> 2) & 1) << 3)     /* 32 floats per lane group */
+#endif
+#elif BV != 1 || !(BN % 64 == 0 || (64 % BN == 0 && BPAD == 0))
 #error "direct-to-LDS tiles: B goes one float per lane; a wavefront covers part of one row, or whole unpadded rows"
 #endif
 #endif
@@ -313,6 +327,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         b_row[e] = q / B_CHUNKS_ROW;
 #if DTL && MODE == 2
         b_col[e] = ACOL(b_row[e], (q % B_CHUNKS_ROW) * BV);
+#elif defined(BSWZ)
+        b_col[e] = ((q % B_CHUNKS_ROW) ^ BSWK(b_row[e])) * BV;
 #else
         b_col[e] = (q % B_CHUNKS_ROW) * BV;
 #endif
@@ -579,6 +595,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if MODE == 2
         const int brow = wn * REP_N * MFMA + li;
         const float* bs = &Bs[buf][brow * SB];
+#elif defined(BSWZ)
+        /* physical column of logical column n in row kb + 4*lg + s: n ^ (lane part) ^ (kb part) */
+        const float* bs = &Bs[buf][(4 * lg) * SB];
+        int bcolx[REP_N];
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j)
+            bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ (MFMA == 16 ? (lg << 4) : (lg << 5));
 #else
         const float* bs = &Bs[buf][(4 * lg) * SB + wn * REP_N * MFMA + li];
 #endif
@@ -601,6 +624,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                 for (int j = 0; j < REP_N; ++j)
 #if MODE == 2
                     b[j] = b4[j][s];
+#elif defined(BSWZ)
+                    b[j] = bs[(kb + s) * SB + (bcolx[j] ^ (MFMA == 16 ? 0 : (((kb >> 2) & 1) << 5)))];
 #else
                     b[j] = bs[(kb + s) * SB + j * MFMA];
 #endif
@@ -661,7 +686,11 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             /* the wavefront's 64 lanes are 64 consecutive columns of one k row */
             const int q0 = e * NT + wv * 64;
             const float* dst = &Bs[buf][(q0 / BN) * SB + (q0 % BN)];
-#if MODE == 0
+#if MODE == 0 && defined(BSWZ)
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * (N * 4));
+#elif MODE == 0
             unsigned vo = b_voff[e];
             if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
             dma4(desc_b, dst, vo, k0 * (N * 4));

@@ -250,6 +250,8 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=5), [0, 8]),               # ragged M, N; padded K
     (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=5, ks=1), [-1, -1]),      # with K streaming
     (96, 144, 128, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=72, st=5), [0, 0]),               # partial last round of chunks
+    (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=5), [0, 0]),               # B in swizzled 16-byte chunks, ragged
+    (256, 256, 512, dict(wm=2, rm=2, wn=2, rn=4, mf=16, bk=32, st=5), [-1, -1]),            # same, 128-wide tile
 ])
 def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
     """Pipeline depth 5: tiles travel global -> LDS without staging registers."""

@@ -72,6 +72,7 @@ def init_arg_parser(parser):
     parser.add_argument("--warm_up", help="warm-up epochs x points, e.g. 4x16", type=str, default="")
     parser.add_argument("--shapes", help="shape table to tune (driver specific)", type=str,
                         default="baseline")
+    parser.add_argument("--cold", help="do not start from the shipped tuned log", action="store_true")
 
 
 def run_driver(args, shapes, make_task, describe):
@@ -99,6 +100,8 @@ def run_driver(args, shapes, make_task, describe):
     if args.warm_up:
         a, b = args.warm_up.lower().split("x")
         kwargs["warm_up"] = (int(a), int(b))
+    if getattr(args, "cold", False):
+        kwargs["warm_start"] = False
     try:
         for i, shape in enumerate(shapes[args.from_:end]):
             print("Optimize %s shape %s [%.6f]" % (describe, str(shape), time.time()), flush=True)

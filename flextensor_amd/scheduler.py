@@ -171,8 +171,10 @@ class Scheduler(object):
         # evaluator(task_key, Config, op_pos, number) -> ms; None = measure on the GPU
         self.evaluator = evaluator
 
+        self.warm_start = True      # seed the search with the shipped log's entry for the task
+        self.resample_rounds = 8    # redraws of random points that the templates refuse
         self.re_evalutate_number = 10
-        self.warm_up_epoch = 20
+        self.warm_up_epoch = 10     # x warm_up_number valid points (refused draws are redrawn)
         self.warm_up_number = 20
         self.verbose = True
         self._pool = None
@@ -216,19 +218,32 @@ class Scheduler(object):
         old_timeout = self.timeout
         while not warm_up_enough:
             for ep in range(warm_up_epoches):
-                warm_up_ret = self.walker_group.forward(warm_up_trials, policy="random")
-                warm_up_configs = [{} for _ in range(warm_up_trials)]
-                warm_up_indices = [{} for _ in range(warm_up_trials)]
-                for count in range(warm_up_trials):
-                    config = warm_up_configs[count]
-                    for type_key in type_keys:
-                        config[type_key] = []
-                        for name in self.space.types[type_key]:
-                            entity = warm_up_ret[name][0][count]
-                            warm_up_indices[count][name] = int(warm_up_ret[name][1][count])
-                            config[type_key].append(entity)
+                warm_up_configs, warm_up_indices = [], []
+                # Random points of the product space are mostly combinations the
+                # templates refuse (the sub-spaces are independent, the constraints
+                # are not): lowering is host-only and cheap, so refused points are
+                # redrawn instead of spending a measurement slot on a certain inf.
+                for attempt in range(self.resample_rounds):
+                    need = warm_up_trials - len(warm_up_configs)
+                    if need <= 0:
+                        break
+                    ret = self.walker_group.forward(need, policy="random")
+                    last_round = attempt == self.resample_rounds - 1
+                    for count in range(need):
+                        config, indices = {}, {}
+                        for type_key in type_keys:
+                            config[type_key] = []
+                            for name in self.space.types[type_key]:
+                                indices[name] = int(ret[name][1][count])
+                                config[type_key].append(ret[name][0][count])
+                        if last_round or self._lowers(configs, config):
+                            warm_up_configs.append(config)
+                            warm_up_indices.append(indices)
+                        else:
+                            self.walker_group.visit.add(str(indices))
+                warm_up_trials_now = len(warm_up_configs)
                 # points already measured are not measured again
-                fresh = [i for i in range(warm_up_trials)
+                fresh = [i for i in range(warm_up_trials_now)
                          if not self.walker_group.ever_met(warm_up_indices[i])]
                 seen = set()
                 uniq = []
@@ -272,7 +287,7 @@ class Scheduler(object):
             pass
         try:
             from .tuned import lookup
-            shipped = lookup(self.task_key)
+            shipped = lookup(self.task_key) if self.warm_start else None
             if shipped is not None and self.op_pos < len(shipped.op_config_lst):
                 candidates.append(shipped.op_config_lst[self.op_pos])
         except Exception:  # noqa: BLE001
@@ -496,6 +511,16 @@ class Scheduler(object):
             best = minimal[0]
         return self.walker_group.to_config(best)
 
+    def _lowers(self, old_configs, config):
+        """True when the templates accept ``config`` in the context of ``old_configs``."""
+        mode = "op" if self.op_pos is not None else "graph"
+        try:
+            cfg, op_pos = self._fetch_config(old_configs, config, mode)
+            schedule_with_config(self.task_key, cfg, op_pos=op_pos, rewrite=self.rewrite)
+            return True
+        except Exception:  # noqa: BLE001
+            return False
+
     # ---- evaluation ----------------------------------------------------
     def _fetch_config(self, old_configs, config, mode):
         if mode == "op":
@@ -704,6 +729,7 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
                                        trial=force_trials[pos], number=number, early_stop=op_stop,
                                        rpc_info=rpc_info, evaluator=evaluator)
             op_scheduler.verbose = verbose
+            op_scheduler.warm_start = bool(kwargs.get("warm_start", True))
             if warm_up:
                 op_scheduler.warm_up_epoch, op_scheduler.warm_up_number = warm_up
             schedulers.append(op_scheduler)

@@ -80,6 +80,20 @@ def run_default_schedule(ops, tensors, stream=0):
     op = ops[0]
     i32 = ctypes.c_int
     out = tensors[-1]
+    if op.kind == "bias_add_nchw":
+        # the stage before it first (into a temporary), then one lane per output adds the bias
+        import torch
+        from .templates import gfx950
+        tmp = torch.empty_like(out)
+        run_default_schedule([op.input_tensors[0].op], list(tensors[:-2]) + [tmp], stream=stream)
+        b, c, h, w = [a.extent for a in op.axis]
+        n = b * c * h * w
+        mod = rt.Module(rt.compile_to_code(gfx950.template_source("elementwise.hip"), []), "bias_add_nchw_f32")
+        mod.launch(_grid1d(n), (256, 1, 1), [rt.ptr(tmp), rt.ptr(tensors[-2]), rt.ptr(out), i32(n), i32(h * w), i32(c)],
+                   stream=stream)
+        torch.cuda.synchronize()
+        mod.close()
+        return
     if op.kind == "gemm":
         if op.attrs.get("transposeA"):
             raise NotImplementedError("transposeA")

@@ -38,6 +38,16 @@ def zero_pad2d(inputs, padding=0):
     return op.output(0)
 
 
+def bias_add_nchw(inputs, bias):
+    """O[b,c,h,w] = I[b,c,h,w] + bias[c]: the stage the reference appends to a
+    convolution that has a bias (flextensor/nn/ops.py:474-478, 673-677)."""
+    if len(bias.shape) != 1 or bias.shape[0] != inputs.shape[1]:
+        raise ValueError("bias must have one entry per output channel")
+    axis = [IterVar(n, e) for n, e in zip("bchw", inputs.shape)]
+    op = ComputeOp("bias", "bias_add_nchw", inputs.shape, inputs.dtype, axis, [], [inputs, bias], {})
+    return op.output(0)
+
+
 def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
     """O[b,k,h,w] = sum_{rc,rw,rh} P[b, (k//Kg)*Cg+rc, h*s+rh*d, w*s+rw*d] * W[k,rc,rh,rw].
 
@@ -45,8 +55,6 @@ def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, grou
     (so the graph is [Padding, conv]); reduce axes are declared [rc, rw, rh];
     out = (in + 2p - d(k-1) - 1)//s + 1.
     """
-    if bias is not None:
-        raise NotImplementedError("bias epilogue is not part of the tuned path")
     batch, in_c, in_h, in_w = inputs.shape
     out_c, c_per_group, k_h, k_w = weight.shape
     if c_per_group * groups != in_c:
@@ -68,6 +76,8 @@ def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, grou
                    [padded, weight],
                    {"stride": stride, "padding": padding, "dilation": dilation,
                     "groups": int(groups), "in_shape": inputs.shape})
+    if bias is not None:
+        return bias_add_nchw(op.output(0), bias)
     return op.output(0)
 
 

@@ -604,8 +604,8 @@ class OpScheduler(Scheduler):
         """Return ``template(op, special, out_name, in_names, materialized_pad)``
         -> list of KernelSpec for this target."""
         if target == "rocm":
-            def template(op, special, out_name, in_names, materialized_pad=False):
-                return gfx950.lower(op, config, special, out_name, in_names, materialized_pad)
+            def template(op, special, out_name, in_names, materialized_pad=False, bias_name=None):
+                return gfx950.lower(op, config, special, out_name, in_names, materialized_pad, bias_name)
             return template
         raise RuntimeError("Currently no support for target %s" % target)
 
@@ -808,6 +808,19 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
     special = None
     if graph_config is not None and graph_config.get("special") and special_names:
         special = dict(zip(special_names, graph_config["special"]))
+    # ---- graph level: bias stages merged into the producing convolution ---
+    from .space import able_merge
+    merge_flags = None
+    if graph_config is not None and graph_config.get("merge"):
+        merge_flags = list(graph_config["merge"][0])
+    merged_into = {}          # producer op index -> the bias op merged into it
+    for i, op in enumerate(op_lst):
+        can = able_merge(op, down_graph)
+        want = can if merge_flags is None else (bool(merge_flags[i]) if i < len(merge_flags) else False)
+        if want and not can:
+            raise gfx950.InvalidConfig("op %d cannot be merged into its producer" % i)
+        if want:
+            merged_into[op_lst.index(op.input_tensors[0].op)] = i
 
     # ---- name the buffers ------------------------------------------------
     names = {}
@@ -817,9 +830,15 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
     intermediates = {}
     specs = []
     for i, op in enumerate(op_lst):
-        if op_states[i].inline:
+        if op_states[i].inline or i in merged_into.values():
             continue
         out_t = op.output(0)
+        bias_name = None
+        if i in merged_into:
+            # the convolution writes the bias stage's output and reads its bias
+            bias_op = op_lst[merged_into[i]]
+            out_t = bias_op.output(0)
+            bias_name = names[bias_op.input_tensors[1]]
         if out_t not in names:
             names[out_t] = "tmp%d" % i
             intermediates[names[out_t]] = (out_t.shape, out_t.dtype)
@@ -837,7 +856,7 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
         if config is None or not any(config.get(k) for k in ("spatial", "reduce", "fuse")):
             config = gfx950.default_config(op)
         template = OpScheduler.generate_op_schedule(target, config)
-        specs.extend(template(op, special, names[out_t], in_names, materialized_pad))
+        specs.extend(template(op, special, names[out_t], in_names, materialized_pad, bias_name))
     return KernelPlan(task_key, bufs, specs, intermediates, configs), bufs
 
 

@@ -40,6 +40,18 @@ def able_inline(op, down_graph):
     return is_compute and (not has_reduce) and (not is_output)
 
 
+def able_merge(op, down_graph):
+    """A per-channel bias stage can be merged into the epilogue of the
+    convolution that feeds it, when nothing else reads the convolution."""
+    from .te import ComputeOp
+    if not isinstance(op, ComputeOp) or op.kind != "bias_add_nchw":
+        return False
+    src = op.input_tensors[0]
+    if not isinstance(src.op, ComputeOp) or src.op.kind != "conv2d_nchw":
+        return False
+    return list(down_graph.get(src, [])) == [op]
+
+
 class Space(object):
     valid_type_keys = ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]
 
@@ -431,6 +443,11 @@ def generate_space_inter_op(op_lst, down_graph, force_inline=False, force_merge=
     knobs (flextensor/space.py:435-452)."""
     space = Space()
     space.add_subspace("inline", generate_inline_space(op_lst, down_graph, force_inline), "inline")
+    # the reference declares a "merge" key and leaves it unused (space.py:443-445); here it
+    # decides whether a bias stage runs in the epilogue of the convolution before it
+    mergeable = [i for i, op in enumerate(op_lst) if able_merge(op, down_graph)]
+    if mergeable:
+        space.add_subspace("merge", MergeSpce(mergeable, len(op_lst), force_merge=force_merge), "merge")
     for key, sspace in (special_space or {}).items():
         space.add_subspace(key, sspace, "special")
     return space

@@ -7,6 +7,9 @@
 //   zero_pad2d_f32  P[b][c][h][w] = X[b][c][h-PAD][w-PAD] inside, 0 outside
 //                   (flextensor/nn/ops.py:83-117), used when the graph config
 //                   does not inline the padding into the convolution
+//   bias_add_nchw_f32  O[b][c][h][w] = I[b][c][h][w] + bias[c] (ops.py:474-478),
+//                   used when the graph config does not merge the bias into
+//                   the convolution's epilogue
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -53,3 +56,13 @@ void zero_pad2d_f32(const float* __restrict__ X, float* __restrict__ P)
     P[gid] = ok ? X[(size_t)pl * (CH * CW) + ih * CW + iw] : 0.0f;
 }
 #endif
+
+/* n = total elements, hw = elements per plane, c = channels */
+extern "C" __global__ __launch_bounds__(256)
+void bias_add_nchw_f32(const float* __restrict__ I, const float* __restrict__ bias,
+                       float* __restrict__ O, int n, int hw, int c)
+{
+    const int stride = gridDim.x * 256;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        O[i] = I[i] + bias[(i / hw) % c];
+}

@@ -192,7 +192,7 @@ def generate_space(op):
         return _gemm_space(GemmView(op))
     if op.kind == "depthwise_conv2d_nchw":
         return _depthwise_space(op)
-    if op.kind == "zero_pad2d":
+    if op.kind in ("zero_pad2d", "bias_add_nchw"):
         return Space()
     raise InvalidConfig("no gfx950 template for operator kind %s" % op.kind)
 
@@ -249,8 +249,10 @@ def _one(config, key, n, what):
     return lst
 
 
-def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False):
+def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
     view = GemmView(op)
+    if bias_name is not None and view.mode != 1:
+        raise InvalidConfig("only the convolution has a bias epilogue")
     sp = _one(config, "spatial", 2, op.kind)
     rd = _one(config, "reduce", 1, op.kind)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
@@ -395,6 +397,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
                                 (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
                                 [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
     args = [("buf", a_name), ("buf", b_name), ("buf", out_name)]
+    if bias_name is not None:
+        D.update(HAS_BIAS=1)       # C = A*B + bias[row], added once whatever the K division
     workspace = {}
     if stream_k:
         # balanced K streaming: stream_k workgroups per compute unit share the
@@ -413,6 +417,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False)
         args += [("buf", out_name + "_parts"), ("buf", out_name + "_count")]
     else:
         grid = (gm * gn * splitk * view.groups, 1, 1)
+    if bias_name is not None:
+        args.append(("buf", bias_name))
     specs.append(KernelSpec("igemm_f32.hip", "igemm_f32", D, grid, (nt * waves_k, 1, 1), args,
                             workspace=workspace))
     return specs
@@ -493,10 +499,24 @@ def _lower_pad(op, out_name, in_names):
                        (256, 1, 1), [("buf", in_names[0]), ("buf", out_name)])]
 
 
-def lower(op, config, special, out_name, in_names, materialized_pad=False):
-    """Config of one operator -> list of KernelSpec (raises InvalidConfig)."""
+def _lower_bias(op, out_name, in_names):
+    b, c, h, w = [x.extent for x in op.axis]
+    n = b * c * h * w
+    return [KernelSpec("elementwise.hip", "bias_add_nchw_f32", {},
+                       (min(ceil_div(n, 256), 4096), 1, 1), (256, 1, 1),
+                       [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name),
+                        ("i32", n), ("i32", h * w), ("i32", c)])]
+
+
+def lower(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
+    """Config of one operator -> list of KernelSpec (raises InvalidConfig).
+    ``bias_name``: buffer of a per-channel bias merged into the epilogue."""
     if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
-        return _lower_gemm(op, config, special, out_name, in_names, materialized_pad)
+        return _lower_gemm(op, config, special, out_name, in_names, materialized_pad, bias_name)
+    if bias_name is not None:
+        raise InvalidConfig("operator kind %s has no bias epilogue" % op.kind)
+    if op.kind == "bias_add_nchw":
+        return _lower_bias(op, out_name, in_names)
     if op.kind == "depthwise_conv2d_nchw":
         return _lower_depthwise(op, config, special, out_name, in_names, materialized_pad)
     if op.kind == "zero_pad2d":

@@ -30,6 +30,9 @@
 //                   WAVES_M*WAVES_N wavefronts each multiply their own K slice
 //                   through their own LDS tiles; the partial tiles are summed
 //                   through LDS at the end (no atomics, no zero fill)
+//   HAS_BIAS        1: C[m][n] = sum + bias[m] (the per-output-channel bias of a
+//                   convolution, flextensor/nn/ops.py:474-478), added exactly
+//                   once whichever way K is divided
 //   DTL             1: tiles travel global -> LDS directly (buffer loads with
 //                   the lds modifier): no staging registers and no LDS store
 //                   instructions. A (and B^T) in 16-byte chunks, 64 per
@@ -82,6 +85,11 @@
 #define BPAD FT_BPAD
 #define AV FT_AV
 #define BV FT_BV
+#ifdef FT_HAS_BIAS
+#define HAS_BIAS FT_HAS_BIAS
+#else
+#define HAS_BIAS 0
+#endif
 #ifdef FT_DTL
 #define DTL FT_DTL
 #else
@@ -283,6 +291,9 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if SK_PER > 0
                , float* sk_part, unsigned* sk_cnt
 #endif
+#if HAS_BIAS
+               , const float* __restrict__ bias
+#endif
                )
 {
     __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
@@ -345,7 +356,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     };
     acc_t acc[REP_M][REP_N];
     /* accumulators -> C for the tile at (m0_, n0_) of group gi_ */
-    auto store_c = [&](int m0_, int n0_, int gi_) {
+    auto store_c = [&](int m0_, int n0_, int gi_, bool first_k_part) {
 #pragma unroll
         for (int i = 0; i < REP_M; ++i) {
 #pragma unroll
@@ -373,10 +384,14 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #else
                         float* dst = C + (size_t)m * N + n;
 #endif
+                        float val = acc[i][j][v];
+#if HAS_BIAS
+                        if (first_k_part) val += bias[gi_ * M + m];
+#endif
 #if SPLITK > 1
-                        unsafeAtomicAdd(dst, acc[i][j][v]);
+                        unsafeAtomicAdd(dst, val);
 #else
-                        *dst = acc[i][j][v];
+                        *dst = val;
 #endif
                     }
                 }
@@ -814,7 +829,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             if (all_in) {
                 add_slots(tile, wg_first + 1, wg_last);
                 if (tid == 0) atomicExch(&sk_cnt[tile], 0u);   /* ready for the next launch */
-                store_c(m0, n0, gi);
+                store_c(m0, n0, gi, true);
                 continue;
             }
         }
@@ -843,7 +858,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         add_slots(tile, wg_first, wg_last);
     }
 #endif
-    store_c(m0, n0, gi);
+    store_c(m0, n0, gi, kz == 0);
     }   /* tile / segment */
 #if SK_PER > 0
     if (check_tile >= 0) {
@@ -859,7 +874,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             add_slots(check_tile, wg_first, wg_last);
             int m0, n0;
             tile_origin(check_tile % (TILES_M * TILES_N), m0, n0);
-            store_c(m0, n0, check_tile / (TILES_M * TILES_N));
+            store_c(m0, n0, check_tile / (TILES_M * TILES_N), true);
         }
     }
 #endif

@@ -186,6 +186,11 @@ def conv2d_nchw_np(x, wt, stride=1, padding=0, dilation=1, groups=1):
     return out
 
 
+def bias_add_nchw_np(y, bias):
+    """O[b,c,h,w] = I[b,c,h,w] + bias[c] in fp32 (flextensor/nn/ops.py:474-478)."""
+    return (np.asarray(y, np.float32) + np.asarray(bias, np.float32)[None, :, None, None]).astype(np.float32)
+
+
 def depthwise_nchw_np(x, wt, stride=1, padding=0, dilation=1):
     x = np.asarray(x, dtype=np.float64)
     wt = np.asarray(wt, dtype=np.float64)

@@ -309,6 +309,50 @@ def test_conv2d_direct_to_lds(oracle, args, kn, pad):
         assert rel(out, ref) <= TOL, inline
 
 
+def _conv_bias(N, C, H, W, K, k, stride=1, padding=0, dilation=1, groups=1):
+    from flextensor_amd.nn import conv2d_nchw
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((K, C // groups, k, k), name="W")
+    bias = placeholder((K,), name="bias")
+    Out = conv2d_nchw(Img, Wt, bias, stride=stride, padding=padding, dilation=dilation, groups=groups)
+    return [Out.op], [Img, Wt, bias, Out]
+
+
+@pytest.mark.parametrize("args,kn,pad", [
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=16), [4, -1]),
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=16, sk=3), [4, -1]),          # grid split-K: bias once
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=32, sk=2, wk=1, st=4), [4, -1]),   # in-workgroup split
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, ks=1, st=5), [0, 0]),      # groups, K streaming, straight into LDS
+    ((4, 6, 7, 7, 9, 3, 2, 1, 2, 3), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16), [4, -1]),                    # the reference's test case
+])
+def test_conv2d_with_bias(oracle, args, kn, pad):
+    """[Padding, conv, bias]: bias merged into the convolution's epilogue, and as its own kernel."""
+    register(_conv_bias, "conv2d", "bias", args, "rocm", 0)
+    key = key_of("conv2d", "bias", args)
+    TASK_TABLE[key].set_specific_space("lds_pad", "enum", [pad])
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w, bias = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    ref = oracle.bias_add_nchw_np(oracle.conv2d_nchw_c(x, w, st, pd, dl, g), bias)
+    M, N, K = ko // g, nb * ref.shape[2] * ref.shape[3], (c // g) * ks * ks
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    cfg = gcfg(M, N, kp, **kn)
+    for merge in ([0, 0, 1], [0, 0, 0]):
+        gc = {k: [] for k in KEYS}
+        gc["inline"], gc["merge"], gc["special"] = [[1, 0, 0]], [merge], [pad]
+        configs = Config([{k: [] for k in KEYS}, cfg, {k: [] for k in KEYS}], gc)
+        s, _ = schedule_with_config(key, configs)
+        assert ("bias_add_nchw_f32" in [x_.kernel for x_ in s.specs]) == (merge[2] == 0)
+        out = run_plan(key, configs, [x, w, bias])
+        assert rel(out, ref) <= TOL, merge
+    # the default-schedule kernels of the three-stage graph
+    dev = [torch.from_numpy(a).cuda() for a in (x, w, bias)]
+    out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+    run_default_schedule(ops, dev + [out], stream=current_stream())
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), ref) <= TOL
+
+
 def test_gemm_transpose_b_vs_oracle(oracle):
     def wrap(M, K, N):
         A = placeholder((M, K), name="A")

@@ -145,6 +145,53 @@ def test_k_streaming_lowering():
         schedule_with_config(I8, Config([i8], None))
 
 
+def _conv_bias(N, C, H, W, K, k, stride=1, padding=0, dilation=1, groups=1):
+    from flextensor_amd.nn import conv2d_nchw
+    from flextensor_amd.te import placeholder
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((K, C // groups, k, k), name="W")
+    bias = placeholder((K,), name="bias")
+    Out = conv2d_nchw(Img, Wt, bias, stride=stride, padding=padding, dilation=dilation, groups=groups)
+    return [Out.op], [Img, Wt, bias, Out]
+
+
+def test_bias_stage_merges_into_the_convolution_or_runs_alone():
+    """Graph [Padding, conv, bias]: the "merge" key decides between a bias
+    epilogue in the convolution kernel and a separate elementwise kernel."""
+    from flextensor_amd.task import register
+    from flextensor_amd.space import generate_space_inter_op
+    args = (2, 16, 14, 14, 32, 3, 1, 1, 1, 1)
+    register(_conv_bias, "conv2d", "bias", args, "rocm", 0)
+    key = Task("conv2d", "bias", None, args, "rocm", 0).key
+    ops, bufs = _conv_bias(*args)
+    op_lst, down = flatten_graph(ops)
+    assert [o.kind for o in op_lst] == ["zero_pad2d", "conv2d_nchw", "bias_add_nchw"]
+    gs = generate_space_inter_op(op_lst, down)
+    assert gs.subspaces["merge"].static_entities == [[0, 0, 1], [0, 0, 0]] or \
+        sorted(gs.subspaces["merge"].static_entities) == [[0, 0, 0], [0, 0, 1]]
+    # default: merged -> one kernel with the bias as fourth buffer
+    s, _ = schedule_with_config(key, Config([], None))
+    assert [x.kernel for x in s.specs] == ["igemm_f32"]
+    assert s.specs[0].defines["HAS_BIAS"] == 1 and [a[1] for a in s.specs[0].args] == ["in1", "in0", "out", "in2"]
+    # not merged -> convolution into a temporary, then the bias kernel
+    g = {k: [] for k in ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]}
+    g["inline"], g["merge"] = [[1, 0, 0]], [[0, 0, 0]]
+    s, _ = schedule_with_config(key, Config([], g))
+    assert [x.kernel for x in s.specs] == ["igemm_f32", "bias_add_nchw_f32"]
+    assert "HAS_BIAS" not in s.specs[0].defines and s.specs[0].args[2] == ("buf", "tmp1")
+    assert [a[1] for a in s.specs[1].args[:3]] == ["tmp1", "in2", "out"] and "tmp1" in s.intermediates
+    # a flag on an op that cannot merge is refused
+    g["merge"] = [[0, 1, 0]]
+    with pytest.raises(gfx950.InvalidConfig):
+        schedule_with_config(key, Config([], g))
+    # the search handles the three-op graph (host cost: fewer kernels is cheaper)
+    np.random.seed(5)
+    s, bufs2, configs = schedule(key, op_trial=2, graph_trial=2, parallel=2, warm_up=(1, 4), verbose=False,
+                                 evaluator=lambda k, c, p, n: 1.0 + len(schedule_with_config(k, c, op_pos=p)[0].specs))
+    assert len(configs.op_config_lst) == 3 and configs.graph_config["merge"][0] == [0, 0, 1]
+    assert [x.kernel for x in s.specs] == ["igemm_f32"]
+
+
 def test_lds_budget_respected_over_whole_space():
     ops, _ = TASK_TABLE[I8].func(*TASK_TABLE[I8].args)
     op_lst, down = flatten_graph(ops)

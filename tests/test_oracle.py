@@ -87,6 +87,23 @@ def test_conv2d_vs_torch(oracle):
         assert rel(oracle.conv2d_nchw_np(x, wt, st, p, d, g), ref) < 1e-12
 
 
+def test_conv2d_bias_vs_torch(oracle):
+    """conv + per-channel bias, as the reference's own test runs it
+    (flextensor/test/test_ops.py:85-115 passes a bias to both sides)."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, (4, 6, 7, 7)).astype(np.float32)
+    w = rng.uniform(-1, 1, (9, 2, 3, 3)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (9,)).astype(np.float32)
+    ref = torch.nn.functional.conv2d(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(bias),
+                                     stride=2, padding=1, dilation=2, groups=3).numpy()
+    got = oracle.bias_add_nchw_np(oracle.conv2d_nchw_c(x, w, 2, 1, 2, 3), bias)
+    assert np.max(np.abs(got - ref)) <= 1e-5 * np.max(np.abs(ref))
+    # the bias alone: a zero image gives bias[c] everywhere
+    z = oracle.bias_add_nchw_np(oracle.conv2d_nchw_c(np.zeros_like(x), w, 2, 1, 2, 3), bias)
+    assert np.array_equal(z, np.broadcast_to(bias[None, :, None, None], z.shape))
+
+
 def test_conv2d_linearity_and_delta(oracle):
     rng = np.random.default_rng(2)
     x1 = rng.uniform(-1, 1, (1, 3, 6, 6)).astype(np.float32)

@@ -168,6 +168,34 @@ def cpu_baseline_for(name, key, ops, budget_s):
     return ms, threads, sample
 
 
+def cpu_naive_for(name, key):
+    """One pass of the default-schedule loop nest (what `create_schedule` + an
+    llvm build gives before any tuning) on ONE host thread: the oracle's plain C
+    restatement. The int8 GEMM is timed on 32 output rows and scaled.
+    Returns (ms per full pass, sample description)."""
+    import numpy as np
+    from flextensor_amd.measure import seeded_inputs
+    from flextensor_amd.task import TASK_TABLE
+    from oracle import oracle as o  # CPU baseline leg only
+    task = TASK_TABLE[key]
+    _, bufs = task.func(*task.args)
+    host = seeded_inputs(bufs, 0)
+    a = task.args
+    frac, sample = 1.0, "one pass of the full workload"
+    t0 = time.perf_counter()
+    if name.startswith("gemm_f32"):
+        o.gemm_f32_c(host[0], host[1])
+    elif name.startswith("gemm_i8"):
+        rows = 32
+        frac, sample = rows / bufs[-1].shape[0], "the first %d output rows, scaled to the full matrix" % rows
+        o.gemm_i8_c(host[0], host[1], 0, rows)
+    elif name.startswith("conv2d"):
+        o.conv2d_nchw_c(host[0], host[1], a[6], a[7], a[8], a[9])
+    else:
+        o.depthwise_nchw_c(host[0], host[1], a[6], a[7], a[8])
+    return (time.perf_counter() - t0) * 1e3 / frac, sample
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,16 +283,20 @@ def main():
     cpu = None
     if not args.no_cpu:
         ms, threads, sample = cpu_baseline_for(name, key, ops, args.cpu_seconds)
+        naive_ms, naive_sample = cpu_naive_for(name, key)
         cpu = {"value": ops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "cores": threads,
                "kind": "port", "ms": ms, "sample": sample + " (oracle/cpu_baseline.c, the "
-               "reference's llvm template structure in C/OpenMP; TVM itself is unavailable)"}
+               "reference's llvm template structure in C/OpenMP; TVM itself is unavailable)",
+               "naive_1thread_ms": naive_ms, "naive_sample": naive_sample + " (oracle/oracle.c, the "
+               "default-schedule loop nest on one thread)"}
         if not args.only_headline:
             for entry, (wname, wkey, wops, _, _, _) in zip(per_config, WORKLOADS):
                 if wname == name:
-                    entry["cpu_ms"], entry["cpu_cores"] = ms, threads
+                    entry["cpu_ms"], entry["cpu_cores"], entry["cpu_naive_1thread_ms"] = ms, threads, naive_ms
                     continue
                 cms, cth, _ = cpu_baseline_for(wname, wkey, wops, 1.0)
                 entry["cpu_ms"], entry["cpu_cores"] = cms, cth
+                entry["cpu_naive_1thread_ms"] = cpu_naive_for(wname, wkey)[0]
 
     line = {
         "metric": "best-config TFLOPS + % of MI355X roofline per op vs CPU llvm baseline",

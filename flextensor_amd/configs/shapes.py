@@ -7,6 +7,10 @@ the same way:
                                                           configs/conv2d_config.py:19
   depthwise  (batch, C, H, W, factor, kh, kw, stride, pad, dilation)
                                                           configs/depthwise_config.py:1-9
+  grouped / dilation
+             (batch, C, H, W, K, kh, kw, stride, pad, dilation, groups)
+                                                          configs/grouped_config.py:1-6,
+                                                          configs/dilation_config.py:8-24
 """
 
 
@@ -39,6 +43,13 @@ depthwise_shapes = [
     (1, 96, 14, 14, 6, 3, 3, 2, 1, 1),
     (1, 160, 7, 7, 6, 3, 3, 1, 1, 1),
 ]
+
+# 1x1 convolution 1024 -> 512 on 14x14 with 4..32 groups
+grouped_shapes = [(1, 1024, 14, 14, 512, 1, 1, 1, 0, 1, g) for g in (4, 8, 16, 32)]
+
+# YOLO layers 5..15 with dilation 2 (same padding as the undilated layers)
+dilation_shapes = [(1, c, hw, hw, k, ks, ks, st, pd, 2, 1)
+                   for (c, hw, k, ks, st, pd) in _yolo_layers[4:]]
 
 # The five benchmark configurations of this backend (index = config number):
 #   gemm fp32 1024^3 | conv 1x64x56x56->64 3x3 | conv 8x256x14x14->512 3x3 and

@@ -11,7 +11,7 @@ should be tunable is registered at import time, here for target ``"rocm"``.
 from .nn import conv2d_nchw, depthwise_conv2d_nchw, gemm as op_gemm, gemm_int8 as op_gemm_int8
 from .space import EnumSpace
 from .te import placeholder
-from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8,
+from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8, grouped_shapes, dilation_shapes,
                              depthwise_shapes, baseline_conv_shapes, baseline_depthwise_shapes,
                              baseline_gemm_shapes, baseline_gemm_int8_shapes)
 
@@ -117,6 +117,12 @@ def _register_all():
                 batch, in_c, h, w, out_c, _, k_h, k_w, _, stride, pad, dil, groups = shape
                 register(conv2d, "conv2d", name + str(i),
                          (batch, in_c, h, w, out_c, k_h, stride, pad, dil, groups),
+                         ROCM_TARGET, j)
+        # flextensor/task.py:436-478
+        for name, shapes in (("grouped", grouped_shapes), ("dilation", dilation_shapes)):
+            for shape in shapes:
+                batch, in_c, h, w, out_c, k, _, stride, pad, dil, groups = shape
+                register(conv2d, "conv2d", name, (batch, in_c, h, w, out_c, k, stride, pad, dil, groups),
                          ROCM_TARGET, j)
         for shape in depthwise_shapes + baseline_depthwise_shapes:
             batch, in_c, h, w, factor, k_h, k_w, stride, pad, dil = shape

@@ -627,6 +627,27 @@ def test_full_size_gemm_int8_bit_exact(oracle):
 
 # --------------------------------------------------- measure / search path --
 
+def _registered_layer_keys():
+    keys = [k for k, t in TASK_TABLE.items() if t.dev_id == 0 and t.target == "rocm" and t.category == "conv2d"
+            and not k.startswith("conv2d_t_") and not k.startswith("conv2d_bias") and not k.startswith("conv2d_smoke")]
+    # yolo at batch 8 repeats the batch-1 layers with 8x the work: keep every third of them
+    b8 = [k for k in keys if k.startswith("conv2d_yolo_b8")]
+    keys = [k for k in keys if not k.startswith("conv2d_yolo_b8")] + b8[::3]
+    return sorted(keys) + ["gemm_gemm_(32, 32, 32)_rocm(0)", "gemm_gemm_(4096, 32, 64)_rocm(0)",
+                           "gemm_gemm_(64, 4096, 4096)_rocm(0)", "gemm_gemm_(2048, 2048, 2048)_rocm(0)"]
+
+
+@pytest.mark.parametrize("key", _registered_layer_keys())
+def test_registered_tasks_default_config_passes_the_gate(key):
+    """Every registered convolution layer (YOLO, grouped, dilated, depthwise,
+    the benchmark shapes) and a few GEMM shapes: the untuned plan matches the
+    default-schedule kernels on the device."""
+    s, bufs = schedule_with_config(key, Config([], None))
+    s.compile()                                   # from the on-disk cache when built ahead of time
+    ms = Measurer(key).evaluate(s, number=3, warmup=1, warm_ms=0)
+    assert 0 < ms < 1e3
+
+
 def test_correctness_gate_rejects_wrong_output():
     key = "gemm_gemm_(256, 256, 256)_rocm(0)"
     m = Measurer(key)

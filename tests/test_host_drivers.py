@@ -37,6 +37,10 @@ def test_driver_keys_are_registered():
     for i, s in enumerate(optimize_conv2d.SHAPES["baseline"]):
         task, trials = mk(i, s, a)
         assert task.key in TASK_TABLE and len(trials) == 2
+    for table in ("grouped", "dilation"):
+        mk = optimize_conv2d.make_task_for(table)
+        for i, shp in enumerate(optimize_conv2d.SHAPES[table]):
+            assert mk(i, shp, a)[0].key in TASK_TABLE, (table, i)
     mk = optimize_conv2d.make_task_for("yolo")
     assert mk(3, optimize_conv2d.SHAPES["yolo"][3], a)[0].key in TASK_TABLE
     for i, s in enumerate(optimize_depthwise_conv2d.SHAPES["baseline"] + optimize_depthwise_conv2d.SHAPES["mobile"]):

@@ -94,6 +94,14 @@ def run_default_schedule(ops, tensors, stream=0):
         torch.cuda.synchronize()
         mod.close()
         return
+    if op.kind == "batch_gemm":
+        nb, M, N = [a.extent for a in op.axis]
+        K = op.reduce_axis[0].extent
+        for b in range(nb):
+            args = [rt.ptr(tensors[0][b]), rt.ptr(tensors[1][b]), rt.ptr(out[b]), i32(M), i32(N), i32(K),
+                    i32(1 if op.attrs.get("transposeB") else 0)]
+            _naive("gemm_f32_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
+        return
     if op.kind == "gemm":
         if op.attrs.get("transposeA"):
             raise NotImplementedError("transposeA")

@@ -130,6 +130,29 @@ def gemm(A, B, transposeA=False, transposeB=False):
     return op.output(0)
 
 
+def batch_gemm(A, B, transposeA=False, transposeB=False):
+    """C[b,i,j] = sum_k A[b,i,k] * B[b,k,j] (B optionally stored [b,j,k]).
+
+    Follows flextensor/nn/ops.py:1111-1158.
+    """
+    if transposeA:
+        raise NotImplementedError("transposeA is not on the tuned path")
+    if A.shape[0] != B.shape[0]:
+        raise ValueError("batch extents differ: %d vs %d" % (A.shape[0], B.shape[0]))
+    batch, m, k_a = A.shape
+    if transposeB:
+        _, n, k_b = B.shape
+    else:
+        _, k_b, n = B.shape
+    if k_a != k_b:
+        raise ValueError("reduce extents differ: %d vs %d" % (k_a, k_b))
+    axis = [IterVar("b", batch), IterVar("i", m), IterVar("j", n)]
+    raxis = [IterVar("k", k_a, "reduce")]
+    op = ComputeOp("compute", "batch_gemm", (batch, m, n), A.dtype, axis, raxis, [A, B],
+                   {"transposeA": False, "transposeB": bool(transposeB)})
+    return op.output(0)
+
+
 def gemm_int8(A, B):
     """C[i,j] = sum_k int32(A[i,k]) * int32(B[j,k]); A [n,l], B [m,l] int8, C int32.
 

@@ -84,12 +84,21 @@ def gemm_int8(N, K, M):
     return [Output.op], [A, B, Output]
 
 
+def batch_gemm(B, N, K, M):
+    """A batch of B products [N,K] x [K,M] (flextensor/nn/ops.py:1111-1158); bufs = [A, B, C]."""
+    from .nn import batch_gemm as op_batch_gemm
+    A = placeholder((B, N, K), name="A")
+    Bm = placeholder((B, K, M), name="B")
+    C = op_batch_gemm(A, Bm)
+    return [C.op], [A, Bm, C]
+
+
 def _attach_default_knobs(task):
     """Give a rocm task the enumerated knobs of its operator family."""
     if task.target != ROCM_TARGET or task.func is None:
         return
     from .templates.gfx950 import special_knobs
-    kind = {gemm: "gemm", gemm_int8: "gemm_int8", conv2d: "conv2d_nchw",
+    kind = {gemm: "gemm", batch_gemm: "batch_gemm", gemm_int8: "gemm_int8", conv2d: "conv2d_nchw",
             depthwise_conv2d: "depthwise_conv2d_nchw"}.get(task.func)
     if kind is None:
         return

@@ -101,6 +101,13 @@ class GemmView(object):
             self.K = op.reduce_axis[0].extent
             self.mode = 2 if op.attrs.get("transposeB") else 0
             self.dtype = "float32"
+        elif kind == "batch_gemm":
+            # one GEMM per batch entry: the batch index is the group index of the kernel
+            self.groups = op.axis[0].extent
+            self.M, self.N = op.axis[1].extent, op.axis[2].extent
+            self.K = op.reduce_axis[0].extent
+            self.mode = 2 if op.attrs.get("transposeB") else 0
+            self.dtype = "float32"
         elif kind == "gemm_int8":
             self.M, self.N = op.axis[0].extent, op.axis[1].extent
             self.K = op.reduce_axis[0].extent
@@ -188,7 +195,7 @@ def _depthwise_space(op):
 
 def generate_space(op):
     """Schedule space of one operator for gfx950."""
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
         return _gemm_space(GemmView(op))
     if op.kind == "depthwise_conv2d_nchw":
         return _depthwise_space(op)
@@ -223,7 +230,7 @@ PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7:
 def special_knobs(kind):
     """Enumerated knobs a task of this operator kind carries by default; they
     are attached with Task.set_specific_space and searched at graph level."""
-    if kind in ("gemm", "conv2d_nchw"):
+    if kind in ("gemm", "conv2d_nchw", "batch_gemm"):
         return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
         return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
@@ -391,6 +398,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         a_name, b_name = in_names[1], in_names[0]
     else:
         a_name, b_name = in_names[0], in_names[1]
+        if view.groups > 1:
+            D.update(CG=view.groups)      # batched GEMM
     if splitk > 1:
         nout = view.M * view.N * view.groups
         specs.append(KernelSpec("elementwise.hip", "fill_zero_f32", {},
@@ -511,7 +520,7 @@ def _lower_bias(op, out_name, in_names):
 def lower(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
     """Config of one operator -> list of KernelSpec (raises InvalidConfig).
     ``bias_name``: buffer of a per-channel bias merged into the epilogue."""
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
         return _lower_gemm(op, config, special, out_name, in_names, materialized_pad, bias_name)
     if bias_name is not None:
         raise InvalidConfig("operator kind %s has no bias epilogue" % op.kind)
@@ -536,7 +545,7 @@ def default_config(op):
     """A reasonable untuned config: what schedule_with_config falls back to
     when a task has no tuned entry, and the seed point of the search."""
     cfg = _empty_config()
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw"):
+    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
         view = GemmView(op)
         i8 = view.dtype == "int8"
 

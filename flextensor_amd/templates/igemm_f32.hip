@@ -7,6 +7,7 @@
 //                             (flextensor/nn/ops.py:1105-1108)
 //   MODE 2  dense GEMM, B^T   A row-major [M][K], B stored [N][K]
 //                             (the transposeB branch, ops.py:1101-1104)
+//           MODE 0 and 2 also run a batch of CG such GEMMs (ops.py:1111-1158)
 //   MODE 1  conv2d NCHW       A = weight [Kout][C*R*S], B = im2col gather of
 //                             the input with zero padding folded into the
 //                             load predicate, N = batch*OH*OW
@@ -275,9 +276,15 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #error "conv mode gathers scalars: BV must be 1"
 #endif
 #else
+/* a batch of independent GEMMs (flextensor/nn/ops.py:1111-1158) reuses the
+ * group index: operand b of every matrix starts b*M*K, b*K*N, b*M*N floats in */
+#ifdef FT_CG
+#define CG FT_CG
+#else
 #define CG 1
-#define A_BYTES (M * K * 4)
-#define B_BYTES (K * N * 4)
+#endif
+#define A_BYTES (CG * M * K * 4)
+#define B_BYTES (CG * K * N * 4)
 #endif
 
 #define A_FLOATS (BM * SA)
@@ -382,7 +389,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if MODE == 1
                         float* dst = C + cbase + (size_t)m * OHW;
 #else
-                        float* dst = C + (size_t)m * N + n;
+                        float* dst = C + ((size_t)gi_ * M + m) * N + n;
 #endif
                         float val = acc[i][j][v];
 #if HAS_BIAS
@@ -525,11 +532,11 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if MODE == 2
         const int n = n0 + b_row[e];
         if (N % BN != 0) ok = ok && (n < N);
-        b_voff[e] = ok ? (unsigned)(n * K + b_col[e]) * 4u : OOB;
+        b_voff[e] = ok ? (unsigned)((gi * N + n) * K + b_col[e]) * 4u : OOB;
 #elif MODE == 0
         const int n = n0 + b_col[e];
         if (N % BN != 0) ok = ok && (n < N);
-        b_voff[e] = ok ? (unsigned)(b_row[e] * N + n) * 4u : OOB;
+        b_voff[e] = ok ? (unsigned)((gi * K + b_row[e]) * N + n) * 4u : OOB;
 #elif KHOIST
         const int cl = b_row[e] / (CR * CS);
         const int rs = b_row[e] % (CR * CS);

@@ -353,6 +353,36 @@ def test_conv2d_with_bias(oracle, args, kn, pad):
     assert rel(out.cpu().numpy(), ref) <= TOL
 
 
+@pytest.mark.parametrize("args,kn,pad", [
+    ((5, 96, 80, 67), dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=16), [4, -1]),                  # ragged, scalar B loads
+    ((3, 200, 136, 328), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=3), [-1, -1]),
+    ((4, 128, 256, 128), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, sk=2), [4, -1]),          # grid split-K atomics
+    ((4, 128, 512, 128), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=32, ks=1, st=5), [-1, -1]),   # K streaming, straight into LDS
+    ((7, 64, 64, 64), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=16, sk=2, wk=1), [4, -1]),       # k-groups
+])
+def test_batch_gemm_vs_oracle(oracle, args, kn, pad):
+    """C[b] = A[b] @ B[b]: the batch index is the kernel's group index."""
+    from flextensor_amd.task import batch_gemm
+    register(batch_gemm, "gemm", "batch_gemm", args, "rocm", 0)
+    key = key_of("gemm", "batch_gemm", args)
+    nb, M, K, N = args
+    ops, bufs = TASK_TABLE[key].func(*args)
+    a, b = seeded_inputs(bufs, seed=sum(args))
+    ref = np.stack([oracle.gemm_f32_c(a[i], b[i]) for i in range(nb)])
+    assert rel(ref, np.matmul(a.astype(np.float64), b.astype(np.float64))) <= TOL
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[0]], [pad]
+    for cfg in (Config([], None), Config([gcfg(M, N, kp, **kn)], g)):
+        out = run_plan(key, cfg, [a, b])
+        assert rel(out, ref) <= TOL
+    dev = [torch.from_numpy(x).cuda() for x in (a, b)]
+    out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+    run_default_schedule(ops, dev + [out], stream=current_stream())
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), ref) <= TOL
+
+
 def test_gemm_transpose_b_vs_oracle(oracle):
     def wrap(M, K, N):
         A = placeholder((M, K), name="A")

@@ -192,6 +192,21 @@ def test_bias_stage_merges_into_the_convolution_or_runs_alone():
     assert [x.kernel for x in s.specs] == ["igemm_f32"]
 
 
+def test_batch_gemm_lowers_to_one_launch_over_all_matrices():
+    from flextensor_amd.task import register, batch_gemm
+    args = (6, 128, 96, 192)
+    register(batch_gemm, "gemm", "batch_gemm", args, "rocm", 0)
+    key = Task("gemm", "batch_gemm", None, args, "rocm", 0).key
+    assert "lds_pad" in TASK_TABLE[key].special_space
+    s, bufs = schedule_with_config(key, Config([], None))
+    spec = s.specs[-1]
+    d = spec.defines
+    assert [x.kernel for x in s.specs] == ["igemm_f32"] and d["CG"] == 6 and d["MODE"] == 0
+    assert (d["M"], d["N"], d["K"]) == (128, 192, 96)
+    tiles = math.ceil(128 / (d["WAVES_M"] * d["REP_M"] * d["MFMA"])) * math.ceil(192 / (d["WAVES_N"] * d["REP_N"] * d["MFMA"]))
+    assert spec.grid[0] == tiles * 6 and [b.shape for b in bufs] == [(6, 128, 96), (6, 96, 192), (6, 128, 192)]
+
+
 def test_lds_budget_respected_over_whole_space():
     ops, _ = TASK_TABLE[I8].func(*TASK_TABLE[I8].args)
     op_lst, down = flatten_graph(ops)

@@ -173,6 +173,7 @@ class Scheduler(object):
 
         self.warm_start = True      # seed the search with the shipped log's entry for the task
         self.resample_rounds = 8    # redraws of random points that the templates refuse
+        self.seed_limit = 24        # heuristic points measured before the random warm-up
         self.re_evalutate_number = 10
         self.warm_up_epoch = 10     # x warm_up_number valid points (refused draws are redrawn)
         self.warm_up_number = 20
@@ -282,7 +283,7 @@ class Scheduler(object):
         op = flatten_graph(ops)[0][self.op_pos]
         candidates = []
         try:
-            candidates.append(gfx950.default_config(op))
+            candidates.extend(gfx950.seed_configs(op, limit=self.seed_limit))
         except Exception:  # noqa: BLE001
             pass
         try:
@@ -292,6 +293,7 @@ class Scheduler(object):
                 candidates.append(shipped.op_config_lst[self.op_pos])
         except Exception:  # noqa: BLE001
             pass
+        points = []
         for cfg in candidates:
             indices = {}
             ok = True
@@ -309,13 +311,23 @@ class Scheduler(object):
                         break
                 if not ok:
                     break
-            if not ok or not indices or self.walker_group.ever_met(indices):
+            if not ok or not indices or self.walker_group.ever_met(indices) \
+                    or any(str(indices) == str(p) for p in points):
                 continue
-            res = self.parallel_evaluate(configs, [self.walker_group.to_config(indices)],
+            if not self._lowers(configs, self.walker_group.to_config(indices)):
+                self.walker_group.visit.add(str(indices))
+                continue
+            points.append(indices)
+        if not points:
+            return
+        # one batch: the candidates compile side by side
+        results = self.parallel_evaluate(configs, [self.walker_group.to_config(p) for p in points],
                                          number=self.number)
-            self._log("seed [%.6f] [ %.6f ]" % (time.time(), res[0]))
-            if res[0] < float("inf"):
-                self.walker_group.record(indices, res[0])
+        self.walker_group.add_perf_data(points, results)
+        self._log("seed [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
+        for indices, res in zip(points, results):
+            if res < float("inf"):
+                self.walker_group.record(indices, res)
             else:
                 self.walker_group.visit.add(str(indices))
 

@@ -594,3 +594,53 @@ def default_config(op):
                           [ceil_div(q, tw), 1, 1, tw]]
         cfg["fuse"] = [[4]]
     return cfg
+
+
+def seed_configs(op, limit=24):
+    """Points worth measuring before the random warm-up: the default config
+    and variations of it along the knobs that decided the hand-tuned shapes
+    (tile aspect and MFMA edge, LDS tile extent incl. whole 3x3 windows,
+    pipeline depth incl. tiles straight into LDS, K streaming when the tiles
+    are fewer than the compute units). Only entities of the op's space are
+    produced; points the templates refuse are dropped by the caller."""
+    base = default_config(op)
+    if op.kind not in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
+        return [base]
+    view = GemmView(op)
+    i8 = view.dtype == "int8"
+    out = [base]
+
+    def tile(extent, w, r, mf):
+        return [ceil_div(extent, w * r * mf), w, r, mf]
+
+    if i8:
+        shapes = [((4, 4, 16), (2, 8, 16)), ((4, 4, 16), (4, 4, 16)), ((4, 2, 32), (4, 2, 32))]
+        bks, depths, streams = [128, 64], [7, 6, 2], [0]
+    else:
+        shapes = [((4, 1, 16), (4, 1, 16)), ((4, 1, 32), (2, 1, 32)), ((2, 1, 32), (2, 1, 32)),
+                  ((4, 1, 16), (1, 1, 16)), ((4, 1, 16), (2, 1, 16)), ((2, 2, 16), (4, 1, 16))]
+        bks = [b for b in (144, 72, 64, 48, 32) if b in F32_BK]
+        depths, streams = [5, 3, 2, 1], [0, 1]
+    for (m_w, m_r, mf), (n_w, n_r, _) in shapes:
+        tm, tn = tile(view.M, m_w, m_r, mf), tile(view.N, n_w, n_r, mf)
+        tiles = tm[0] * tn[0] * view.groups
+        for bk in bks:
+            kps = [kp for kp in view.KP_options if kp % bk == 0]
+            if not kps:
+                continue
+            for depth in depths:
+                for stream in streams:
+                    if stream and (i8 or tiles >= 2 * NUM_CUS):
+                        continue
+                    cfg = _empty_config()
+                    cfg["spatial"] = [tm, tn]
+                    cfg["reduce"] = [[1, kps[0] // bk, bk]]
+                    cfg["unroll"] = [[depth, 1]]
+                    cfg["fuse"] = [[8]]
+                    cfg["reorder"] = [[1, 0, stream]]
+                    out.append(cfg)
+    # spread over the variations instead of exhausting the first tile shape
+    if len(out) > limit:
+        step = (len(out) - 1) / float(limit - 1)
+        out = [out[int(round(i * step))] for i in range(limit)]
+    return out

@@ -105,6 +105,19 @@ def kernel_ms(built, m, iters=None, warmup=20):
     return built.time(m.sets, warmup=warmup, iters=iters, warm_ms=WARM_MS), metric
 
 
+def launch_floor_ms():
+    """Mean time per launch of an empty kernel, back to back on the launch
+    stream: what any kernel measured per launch pays before it does work."""
+    from flextensor_amd import runtime as rt
+    from flextensor_amd.plan import current_stream
+    mod = rt.Module.from_source('extern "C" __global__ void ft_empty(int* p) { if (p == nullptr) return; }', "ft_empty")
+    import torch
+    x = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ms = mod.time((256,), (256,), [rt.ptr(x)], warmup=20000, iters=4000, stream=current_stream())
+    mod.close()
+    return ms
+
+
 def copy_yardstick(mib, iters):
     """Time copy_f32 over `mib` MiB (read) + `mib` MiB (write)."""
     import ctypes as ct
@@ -263,6 +276,7 @@ def main():
     roof = roofline(name, bound, dtype, ops, nbytes, k_ms)
     roof["kernel"] = plan.specs[-1].kernel
     roof["kernel_ms"] = k_ms
+    roof["launch_floor_ms"] = launch_floor_ms()
     built.close()
 
     per_config = []

@@ -442,6 +442,13 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     }
 
 #endif
+    /* The last MFMA's result registers may not be read for 19 issue slots
+     * (16 passes) and the hardware does not enforce it; the compiler's hazard
+     * pass can lose a short path through branchy code, so the distance from
+     * the main loop to the first accumulator read is explicit. */
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
 #if CVEC
     /* swapped operands: lane (li, lg) holds C[m = li][n = 4*lg + 0..3] (16x16),

@@ -790,6 +790,15 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         }
     }
 #endif
+    /* A 16-pass MFMA's last result registers may not be read for 19 issue
+     * slots, and nothing in the hardware enforces that. The compiler pads
+     * the code it can follow, but in the segment loop's control flow of
+     * balanced K streaming its hazard pass lost the short path from the last
+     * MFMA to the first accumulator read (a full tile's store then took the
+     * value from before the last MFMA), so the distance is made explicit. */
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
 #if WAVES_K > 1
     /* ---- sum the k-groups' partial tiles through LDS --------------------- */

@@ -293,6 +293,10 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, 8]),      # 1x1, N=392
     ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=16, sk=4, wk=1, st=5), [0, 0]),   # BN=16, 4 k-groups
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=72, sk=2, wk=1, st=5), [0, 0]),   # BN=32, whole windows
+    # K streaming with whole tiles between two shared ones: the tile store reads the
+    # accumulators right after the last MFMA (the store once came 19 issue slots too early)
+    ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64, st=5, ks=1), [-1, 0]),
+    ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=32, st=2, ks=1), [-1, 0]),
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)

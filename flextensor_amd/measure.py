@@ -94,6 +94,32 @@ def run_default_schedule(ops, tensors, stream=0):
         torch.cuda.synchronize()
         mod.close()
         return
+    if op.kind == "col2img_nchw":
+        # im2col, GEMM, (bias,) col2img define the same function as the direct
+        # convolution: one lane per output runs the convolution's own sum
+        import torch
+        from .templates import gfx950
+        stage = op.input_tensors[0].op
+        has_bias = stage.kind == "bias_add_ghw"
+        if has_bias:
+            stage = stage.input_tensors[0].op
+        a = stage.attrs
+        b, ko, p, q = [x.extent for x in op.axis]
+        _, c, h, w = a["in_shape"]
+        r, s = a["kernel"]
+        dst = torch.empty_like(out) if has_bias else out
+        args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(dst)] + [i32(v) for v in (
+            b, c, h, w, ko, r, s, a["stride"][0], a["stride"][1], a["padding"][0], a["padding"][1],
+            a["dilation"][0], a["dilation"][1], a["groups"], p, q)]
+        _naive("conv2d_nchw_naive").launch(_grid1d(b * ko * p * q), (256, 1, 1), args, stream=stream)
+        if has_bias:
+            n = b * ko * p * q
+            mod = rt.Module(rt.compile_to_code(gfx950.template_source("elementwise.hip"), []), "bias_add_nchw_f32")
+            mod.launch(_grid1d(n), (256, 1, 1), [rt.ptr(dst), rt.ptr(tensors[2]), rt.ptr(out), i32(n), i32(p * q), i32(ko)],
+                       stream=stream)
+            torch.cuda.synchronize()
+            mod.close()
+        return
     if op.kind == "batch_gemm":
         nb, M, N = [a.extent for a in op.axis]
         K = op.reduce_axis[0].extent

@@ -108,6 +108,75 @@ def depthwise_conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilati
     return op.output(0)
 
 
+def im2col_nchw_naive(inputs, kernel_size, stride=1, padding=0, dilation=1, groups=1):
+    """col[g, h, w] = P[w // (P*Q), g*Cg + h // (kh*kw),
+                        (w % (P*Q)) // Q * s + (h % (kh*kw)) // kw * d,  w % Q * s + h % kw * d]
+
+    Follows flextensor/nn/ops.py:896-950: the padded image is its own operator;
+    rows are (channel, kh, kw), columns are (batch, out_h, out_w).
+    """
+    batch, in_c, in_h, in_w = inputs.shape
+    out_c, c_per_group, k_h, k_w = [int(x) for x in kernel_size]
+    if c_per_group * groups != in_c:
+        raise ValueError("kernel channels %d * groups %d != input channels %d" % (c_per_group, groups, in_c))
+    if out_c % groups != 0:
+        raise ValueError("output channels not divisible by groups")
+    stride = _pair(stride, "stride")
+    padding = _pair(padding, "padding")
+    dilation = _pair(dilation, "dilation")
+    out_h = (in_h + 2 * padding[0] - dilation[0] * (k_h - 1) - 1) // stride[0] + 1
+    out_w = (in_w + 2 * padding[1] - dilation[1] * (k_w - 1) - 1) // stride[1] + 1
+    padded = zero_pad2d(inputs, padding=padding)
+    out_shape = (groups, k_h * k_w * c_per_group, batch * out_h * out_w)
+    axis = [IterVar(n, e) for n, e in zip("ghw", out_shape)]
+    op = ComputeOp("Img2Col", "im2col_nchw", out_shape, inputs.dtype, axis, [], [padded],
+                   {"stride": stride, "padding": padding, "dilation": dilation, "groups": int(groups),
+                    "in_shape": inputs.shape, "kernel": (k_h, k_w), "out_hw": (out_h, out_w),
+                    "out_channel": out_c})
+    return op.output(0)
+
+
+def col2img_nchw(inputs, P, Q):
+    """O[b, c, h, w] = I[c // Mg, c % Mg, b*(P*Q) + h*Q + w] (flextensor/nn/ops.py:953-979)."""
+    groups, m_per_group, width = inputs.shape
+    if width % (P * Q) != 0:
+        raise ValueError("column count %d is not a multiple of P*Q = %d" % (width, P * Q))
+    out_shape = (width // (P * Q), m_per_group * groups, int(P), int(Q))
+    axis = [IterVar(n, e) for n, e in zip("bchw", out_shape)]
+    op = ComputeOp("Col2Img", "col2img_nchw", out_shape, inputs.dtype, axis, [], [inputs], {})
+    return op.output(0)
+
+
+def gemm_conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, groups=1):
+    """Convolution as an explicit im2col, one GEMM per group and a col2img
+    (flextensor/nn/ops.py:982-1044):
+
+        gemm[g, h, w] = sum_k col[g, k, w] * W[g*Mg + h, k // (kh*kw), (k % (kh*kw)) // kw, k % kw]
+
+    The graph is [Padding, Img2Col, ComputeGemm, (ComputeBias,) Col2Img]; the
+    result equals conv2d_nchw's.
+    """
+    out_c, c_per_group, k_h, k_w = weight.shape
+    if out_c % groups != 0:
+        raise ValueError("output channels not divisible by groups")
+    m_per_group = out_c // groups
+    col = im2col_nchw_naive(inputs, weight.shape, stride, padding, dilation, groups)
+    out_h, out_w = col.op.attrs["out_hw"]
+    _, k_ext, n_ext = col.shape
+    axis = [IterVar("g", groups), IterVar("h", m_per_group), IterVar("w", n_ext)]
+    raxis = [IterVar("k", k_ext, "reduce")]
+    op = ComputeOp("ComputeGemm", "col_gemm", (groups, m_per_group, n_ext), inputs.dtype, axis, raxis,
+                   [col, weight], dict(col.op.attrs))
+    out = op.output(0)
+    if bias is not None:
+        if len(bias.shape) != 1 or bias.shape[0] != out_c:
+            raise ValueError("bias must have one entry per output channel")
+        baxis = [IterVar(n, e) for n, e in zip("ghw", out.shape)]
+        bop = ComputeOp("ComputeBias", "bias_add_ghw", out.shape, out.dtype, baxis, [], [out, bias], {})
+        out = bop.output(0)
+    return col2img_nchw(out, out_h, out_w)
+
+
 def gemm(A, B, transposeA=False, transposeB=False):
     """C[i,j] = sum_k A[i,k] * B[k,j] (operands optionally stored transposed).
 

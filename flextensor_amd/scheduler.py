@@ -616,8 +616,10 @@ class OpScheduler(Scheduler):
         """Return ``template(op, special, out_name, in_names, materialized_pad)``
         -> list of KernelSpec for this target."""
         if target == "rocm":
-            def template(op, special, out_name, in_names, materialized_pad=False, bias_name=None):
-                return gfx950.lower(op, config, special, out_name, in_names, materialized_pad, bias_name)
+            def template(op, special, out_name, in_names, materialized_pad=False, bias_name=None,
+                         through=(), merged_out=None):
+                return gfx950.lower(op, config, special, out_name, in_names, materialized_pad, bias_name,
+                                    through=through, merged_out=merged_out)
             return template
         raise RuntimeError("Currently no support for target %s" % target)
 
@@ -825,14 +827,19 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
     merge_flags = None
     if graph_config is not None and graph_config.get("merge"):
         merge_flags = list(graph_config["merge"][0])
-    merged_into = {}          # producer op index -> the bias op merged into it
+    merged = set()            # stages that run inside their producer's kernel
     for i, op in enumerate(op_lst):
         can = able_merge(op, down_graph)
         want = can if merge_flags is None else (bool(merge_flags[i]) if i < len(merge_flags) else False)
         if want and not can:
             raise gfx950.InvalidConfig("op %d cannot be merged into its producer" % i)
         if want:
-            merged_into[op_lst.index(op.input_tensors[0].op)] = i
+            merged.add(i)
+    for i in merged:
+        # a stage merges into a kernel: a merged stage behind an unmerged one has none
+        src = op_lst.index(op_lst[i].input_tensors[0].op)
+        if op_lst[src].kind in ("bias_add_nchw", "bias_add_ghw") and src not in merged:
+            raise gfx950.InvalidConfig("op %d follows a stage that is not merged" % i)
 
     # ---- name the buffers ------------------------------------------------
     names = {}
@@ -842,33 +849,43 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
     intermediates = {}
     specs = []
     for i, op in enumerate(op_lst):
-        if op_states[i].inline or i in merged_into.values():
+        if op_states[i].inline or i in merged:
             continue
         out_t = op.output(0)
         bias_name = None
-        if i in merged_into:
-            # the convolution writes the bias stage's output and reads its bias
-            bias_op = op_lst[merged_into[i]]
-            out_t = bias_op.output(0)
-            bias_name = names[bias_op.input_tensors[1]]
+        merged_out = None
+        while True:
+            # follow the chain of merged stages: the kernel writes the last one's output
+            users = list(down_graph.get(out_t, []))
+            if len(users) != 1 or op_lst.index(users[0]) not in merged:
+                break
+            stage = users[0]
+            if stage.kind in ("bias_add_nchw", "bias_add_ghw"):
+                bias_name = names[stage.input_tensors[1]]
+            else:
+                merged_out = stage.kind
+            out_t = stage.output(0)
         if out_t not in names:
             names[out_t] = "tmp%d" % i
             intermediates[names[out_t]] = (out_t.shape, out_t.dtype)
         in_names = []
         materialized_pad = False
+        through = []
         for t in op.input_tensors:
             src = t
             # an inlined producer is read through: the consumer sees its input
             while isinstance(src.op, ComputeOp) and op_states[op_lst.index(src.op)].inline:
+                through.append(src.op.kind)
                 src = src.op.input_tensors[0]
-            if isinstance(t.op, ComputeOp) and t.op.kind == "zero_pad2d" and src is t:
+            if isinstance(src.op, ComputeOp) and src.op.kind == "zero_pad2d":
                 materialized_pad = True
             in_names.append(names[src])
         config = op_config_lst[i] if i < len(op_config_lst) and op_config_lst[i] else None
         if config is None or not any(config.get(k) for k in ("spatial", "reduce", "fuse")):
             config = gfx950.default_config(op)
         template = OpScheduler.generate_op_schedule(target, config)
-        specs.extend(template(op, special, names[out_t], in_names, materialized_pad, bias_name))
+        specs.extend(template(op, special, names[out_t], in_names, materialized_pad, bias_name,
+                              through=tuple(through), merged_out=merged_out))
     return KernelPlan(task_key, bufs, specs, intermediates, configs), bufs
 
 

@@ -40,14 +40,23 @@ def able_inline(op, down_graph):
     return is_compute and (not has_reduce) and (not is_output)
 
 
+# stage kind -> producer kinds whose kernel can take the stage over
+MERGE_RULES = {
+    "bias_add_nchw": ("conv2d_nchw",),            # bias in the convolution's epilogue
+    "bias_add_ghw": ("col_gemm",),                # the same for the GEMM of an im2col convolution
+    "col2img_nchw": ("col_gemm", "bias_add_ghw"),  # the GEMM stores NCHW itself
+}
+
+
 def able_merge(op, down_graph):
-    """A per-channel bias stage can be merged into the epilogue of the
-    convolution that feeds it, when nothing else reads the convolution."""
+    """An elementwise stage (per-channel bias, col2img) can be merged into the
+    stores of the kernel that feeds it, when nothing else reads that kernel's
+    output."""
     from .te import ComputeOp
-    if not isinstance(op, ComputeOp) or op.kind != "bias_add_nchw":
+    if not isinstance(op, ComputeOp) or op.kind not in MERGE_RULES:
         return False
     src = op.input_tensors[0]
-    if not isinstance(src.op, ComputeOp) or src.op.kind != "conv2d_nchw":
+    if not isinstance(src.op, ComputeOp) or src.op.kind not in MERGE_RULES[op.kind]:
         return False
     return list(down_graph.get(src, [])) == [op]
 

@@ -67,6 +67,18 @@ def depthwise_conv2d(N, C, H, W, factor, kernel_size, stride=1, padding=0, dilat
     return [Output.op], [Img, Wt, Output]
 
 
+def gemm_conv2d(N, C, H, W, K, kernel_size, stride=1, padding=0, dilation=1, groups=1):
+    """flextensor/task.py:131-135: the convolution as im2col, GEMM, col2img;
+    bufs = [Img, W, Output]. The weight holds C // groups channels per filter
+    (the reference declares all C, which its GEMM stage never reads beyond
+    C // groups and which only agrees with the image for groups = 1)."""
+    from .nn import gemm_conv2d_nchw
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((K, C // groups, kernel_size, kernel_size), name="W")
+    Output = gemm_conv2d_nchw(Img, Wt, stride=stride, padding=padding, dilation=dilation, groups=groups)
+    return [Output.op], [Img, Wt, Output]
+
+
 def gemm(N, K, M):
     """flextensor/task.py:145-149; A [N,K] · B [K,M] -> [N,M], fp32."""
     A = placeholder((N, K), name="A")
@@ -99,7 +111,7 @@ def _attach_default_knobs(task):
         return
     from .templates.gfx950 import special_knobs
     kind = {gemm: "gemm", batch_gemm: "batch_gemm", gemm_int8: "gemm_int8", conv2d: "conv2d_nchw",
-            depthwise_conv2d: "depthwise_conv2d_nchw"}.get(task.func)
+            gemm_conv2d: "col_gemm", depthwise_conv2d: "depthwise_conv2d_nchw"}.get(task.func)
     if kind is None:
         return
     for key, knobs in special_knobs(kind).items():
@@ -127,6 +139,9 @@ def _register_all():
                 register(conv2d, "conv2d", name + str(i),
                          (batch, in_c, h, w, out_c, k_h, stride, pad, dil, groups),
                          ROCM_TARGET, j)
+                # flextensor/task.py:349-366
+                register(gemm_conv2d, "gemm_conv2d", name + str(i),
+                         (batch, in_c, h, w, out_c, k_h, stride, pad, dil, groups), ROCM_TARGET, j)
         # flextensor/task.py:436-478
         for name, shapes in (("grouped", grouped_shapes), ("dilation", dilation_shapes)):
             for shape in shapes:

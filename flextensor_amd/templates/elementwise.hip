@@ -10,6 +10,12 @@
 //   bias_add_nchw_f32  O[b][c][h][w] = I[b][c][h][w] + bias[c] (ops.py:474-478),
 //                   used when the graph config does not merge the bias into
 //                   the convolution's epilogue
+//   im2col_nchw_f32 col[g][k][n] = X[b][g*Cg + c][p*s + r*d - pad][q*s + t*d - pad],
+//                   k = (c, r, t), n = (b, p, q), 0 outside the image
+//                   (ops.py:896-950), used when the graph config does not
+//                   inline the column matrix into the GEMM's loads
+//   col2img_nchw_f32 O[b][c][p][q] = I[c][b*P*Q + p*Q + q] (ops.py:953-979), used
+//                   when the graph config does not merge it into the GEMM's stores
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -66,3 +72,56 @@ void bias_add_nchw_f32(const float* __restrict__ I, const float* __restrict__ bi
     for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
         O[i] = I[i] + bias[(i / hw) % c];
 }
+
+#ifdef FT_COLK
+/* convolution geometry: CB batch, CG groups, CC input channels, CH x CW the
+ * image as stored (already padded when CPAD is 0 and the padding is its own
+ * operator), CR x CS window, CP x CQ output plane, MG output channels per group */
+#define CB FT_CB
+#define CG FT_CG
+#define CC FT_CC
+#define CH FT_CH
+#define CW FT_CW
+#define CR FT_CR
+#define CS FT_CS
+#define CSTR FT_CSTR
+#define CPAD FT_CPAD
+#define CDIL FT_CDIL
+#define CP FT_CP
+#define CQ FT_CQ
+#define MG FT_MG
+#define COL_K ((CC / CG) * CR * CS)
+#define COL_N (CB * CP * CQ)
+extern "C" __global__ __launch_bounds__(256)
+void im2col_nchw_f32(const float* __restrict__ X, float* __restrict__ col)
+{
+    const long long total = (long long)CG * COL_K * COL_N;
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long gid = (long long)blockIdx.x * 256 + threadIdx.x; gid < total; gid += stride) {
+        const int n = (int)(gid % COL_N);
+        const int k = (int)((gid / COL_N) % COL_K);
+        const int g = (int)(gid / ((long long)COL_N * COL_K));
+        const int b = n / (CP * CQ);
+        const int p = (n % (CP * CQ)) / CQ;
+        const int q = n % CQ;
+        const int c = g * (CC / CG) + k / (CR * CS);
+        const int ih = p * CSTR + ((k % (CR * CS)) / CS) * CDIL - CPAD;
+        const int iw = q * CSTR + (k % CS) * CDIL - CPAD;
+        const bool ok = (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+        col[gid] = ok ? X[((size_t)b * CC + c) * (CH * CW) + ih * CW + iw] : 0.0f;
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256)
+void col2img_nchw_f32(const float* __restrict__ I, float* __restrict__ O)
+{
+    const long long total = (long long)CG * MG * COL_N;
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long gid = (long long)blockIdx.x * 256 + threadIdx.x; gid < total; gid += stride) {
+        const int pq = (int)(gid % (CP * CQ));
+        const int c = (int)((gid / (CP * CQ)) % (CG * MG));
+        const int b = (int)(gid / ((long long)(CP * CQ) * (CG * MG)));
+        O[gid] = I[(size_t)c * COL_N + (size_t)b * (CP * CQ) + pq];
+    }
+}
+#endif

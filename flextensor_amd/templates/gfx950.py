@@ -89,7 +89,7 @@ class KernelSpec(object):
 class GemmView(object):
     """M, N, K and addressing mode of a contraction-shaped operator."""
 
-    def __init__(self, op):
+    def __init__(self, op, col_inlined=False):
         kind = op.kind
         self.kind = kind
         self.conv = None
@@ -131,6 +131,25 @@ class GemmView(object):
             self.groups = groups
             self.conv = dict(CB=b, CG=groups, CC=c * groups, CH=h, CW=w, CR=r, CS=s, CSTR=a["stride"][0],
                              CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
+        elif kind == "col_gemm":
+            # the GEMM stage of an im2col convolution: one [Mg,K] x [K,N] product per group.
+            # With the column matrix read through (inlined) it is the implicit GEMM over the
+            # image; otherwise a batch of plain GEMMs over the stored columns.
+            a = op.attrs
+            if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
+                    or a["dilation"][0] != a["dilation"][1]:
+                raise NotImplementedError("anisotropic stride/padding/dilation")
+            groups = op.axis[0].extent
+            self.M, self.N = op.axis[1].extent, op.axis[2].extent
+            self.K = op.reduce_axis[0].extent
+            self.groups = groups
+            self.dtype = "float32"
+            b, cin, h, w = a["in_shape"]
+            r, sw = a["kernel"]
+            p, q = a["out_hw"]
+            self.conv = dict(CB=b, CG=groups, CC=cin, CH=h, CW=w, CR=r, CS=sw, CSTR=a["stride"][0],
+                             CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
+            self.mode = 1 if col_inlined else 0
         else:
             raise InvalidConfig("operator kind %s has no GEMM view" % kind)
         # K as the kernels iterate it: fp32 pads the tail up to a multiple of
@@ -147,6 +166,8 @@ class GemmView(object):
                 self.KP_options.insert(0, self.K)
         self.KP = self.KP_options[-1]
 
+
+GEMM_KINDS = ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm", "col_gemm")
 
 F32_BK = (8, 16, 32, 48, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
 I8_BK = (64, 128, 256)
@@ -195,11 +216,11 @@ def _depthwise_space(op):
 
 def generate_space(op):
     """Schedule space of one operator for gfx950."""
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
+    if op.kind in GEMM_KINDS:
         return _gemm_space(GemmView(op))
     if op.kind == "depthwise_conv2d_nchw":
         return _depthwise_space(op)
-    if op.kind in ("zero_pad2d", "bias_add_nchw"):
+    if op.kind in ("zero_pad2d", "bias_add_nchw", "bias_add_ghw", "im2col_nchw", "col2img_nchw"):
         return Space()
     raise InvalidConfig("no gfx950 template for operator kind %s" % op.kind)
 
@@ -230,7 +251,7 @@ PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7:
 def special_knobs(kind):
     """Enumerated knobs a task of this operator kind carries by default; they
     are attached with Task.set_specific_space and searched at graph level."""
-    if kind in ("gemm", "conv2d_nchw", "batch_gemm"):
+    if kind in ("gemm", "conv2d_nchw", "batch_gemm", "col_gemm"):
         return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
     if kind == "gemm_int8":
         return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
@@ -256,10 +277,15 @@ def _one(config, key, n, what):
     return lst
 
 
-def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
-    view = GemmView(op)
-    if bias_name is not None and view.mode != 1:
+def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None,
+                through=(), merged_out=None):
+    view = GemmView(op, col_inlined="im2col_nchw" in through)
+    if bias_name is not None and view.mode != 1 and op.kind != "col_gemm":
         raise InvalidConfig("only the convolution has a bias epilogue")
+    if merged_out is not None and not (op.kind == "col_gemm" and merged_out == "col2img_nchw"):
+        raise InvalidConfig("stage %s cannot run in the stores of %s" % (merged_out, op.kind))
+    if merged_out is not None and view.mode != 1:
+        raise InvalidConfig("col2img merges into the GEMM that reads the image itself")
     sp = _one(config, "spatial", 2, op.kind)
     rd = _one(config, "reduce", 1, op.kind)
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
@@ -394,10 +420,14 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
             conv["CW"] += 2 * conv["CPAD"]
             conv["CPAD"] = 0
         D.update(conv)
+        if op.kind == "col_gemm" and merged_out is None:
+            D.update(COLOUT=1)            # C stays [groups][M][N] for the col2img stage
         # A = weight, B = image
         a_name, b_name = in_names[1], in_names[0]
     else:
         a_name, b_name = in_names[0], in_names[1]
+        if op.kind == "col_gemm":
+            a_name, b_name = in_names[1], in_names[0]      # A = weight, B = stored columns
         if view.groups > 1:
             D.update(CG=view.groups)      # batched GEMM
     if splitk > 1:
@@ -509,7 +539,12 @@ def _lower_pad(op, out_name, in_names):
 
 
 def _lower_bias(op, out_name, in_names):
-    b, c, h, w = [x.extent for x in op.axis]
+    if op.kind == "bias_add_ghw":
+        # [groups][Mg][N] is one image of groups*Mg channels with N elements each
+        g, mg, hw = [x.extent for x in op.axis]
+        b, c, h, w = 1, g * mg, 1, hw
+    else:
+        b, c, h, w = [x.extent for x in op.axis]
     n = b * c * h * w
     return [KernelSpec("elementwise.hip", "bias_add_nchw_f32", {},
                        (min(ceil_div(n, 256), 4096), 1, 1), (256, 1, 1),
@@ -517,14 +552,57 @@ def _lower_bias(op, out_name, in_names):
                         ("i32", n), ("i32", h * w), ("i32", c)])]
 
 
-def lower(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
+def _conv_defines(attrs, materialized_pad):
+    if attrs["stride"][0] != attrs["stride"][1] or attrs["padding"][0] != attrs["padding"][1] \
+            or attrs["dilation"][0] != attrs["dilation"][1]:
+        raise NotImplementedError("anisotropic stride/padding/dilation")
+    b, cin, h, w = attrs["in_shape"]
+    pad = attrs["padding"][0]
+    if materialized_pad:
+        h, w, pad = h + 2 * pad, w + 2 * pad, 0
+    groups = attrs["groups"]
+    return dict(COLK=1, CB=b, CG=groups, CC=cin, CH=h, CW=w, CR=attrs["kernel"][0], CS=attrs["kernel"][1],
+                CSTR=attrs["stride"][0], CPAD=pad, CDIL=attrs["dilation"][0], CP=attrs["out_hw"][0],
+                CQ=attrs["out_hw"][1], MG=attrs["out_channel"] // groups)
+
+
+def _lower_im2col(op, out_name, in_names, materialized_pad):
+    g, k, n = [x.extent for x in op.axis]
+    total = g * k * n
+    return [KernelSpec("elementwise.hip", "im2col_nchw_f32", _conv_defines(op.attrs, materialized_pad),
+                       (min(ceil_div(total, 256), 16384), 1, 1), (256, 1, 1),
+                       [("buf", in_names[0]), ("buf", out_name)])]
+
+
+def _lower_col2img(op, out_name, in_names):
+    b, c, p, q = [x.extent for x in op.axis]
+    g, mg, _ = op.input_tensors[0].shape
+    # only the output geometry matters to this kernel; the image constants are placeholders
+    D = dict(COLK=1, CB=b, CG=g, CC=g, CH=1, CW=1, CR=1, CS=1, CSTR=1, CPAD=0, CDIL=1, CP=p, CQ=q, MG=mg)
+    total = b * c * p * q
+    return [KernelSpec("elementwise.hip", "col2img_nchw_f32", D,
+                       (min(ceil_div(total, 256), 16384), 1, 1), (256, 1, 1),
+                       [("buf", in_names[0]), ("buf", out_name)])]
+
+
+def lower(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None,
+          through=(), merged_out=None):
     """Config of one operator -> list of KernelSpec (raises InvalidConfig).
-    ``bias_name``: buffer of a per-channel bias merged into the epilogue."""
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
-        return _lower_gemm(op, config, special, out_name, in_names, materialized_pad, bias_name)
+    ``bias_name``: buffer of a per-channel bias merged into the epilogue;
+    ``through``: kinds of the inlined producers the operator reads through;
+    ``merged_out``: kind of a layout stage merged into the operator's stores."""
+    if op.kind in GEMM_KINDS:
+        return _lower_gemm(op, config, special, out_name, in_names, materialized_pad, bias_name,
+                           through, merged_out)
     if bias_name is not None:
         raise InvalidConfig("operator kind %s has no bias epilogue" % op.kind)
-    if op.kind == "bias_add_nchw":
+    if merged_out is not None:
+        raise InvalidConfig("operator kind %s takes no merged stage" % op.kind)
+    if op.kind == "im2col_nchw":
+        return _lower_im2col(op, out_name, in_names, materialized_pad)
+    if op.kind == "col2img_nchw":
+        return _lower_col2img(op, out_name, in_names)
+    if op.kind in ("bias_add_nchw", "bias_add_ghw"):
         return _lower_bias(op, out_name, in_names)
     if op.kind == "depthwise_conv2d_nchw":
         return _lower_depthwise(op, config, special, out_name, in_names, materialized_pad)
@@ -545,7 +623,7 @@ def default_config(op):
     """A reasonable untuned config: what schedule_with_config falls back to
     when a task has no tuned entry, and the seed point of the search."""
     cfg = _empty_config()
-    if op.kind in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
+    if op.kind in GEMM_KINDS:
         view = GemmView(op)
         i8 = view.dtype == "int8"
 
@@ -604,7 +682,7 @@ def seed_configs(op, limit=24):
     are fewer than the compute units). Only entities of the op's space are
     produced; points the templates refuse are dropped by the caller."""
     base = default_config(op)
-    if op.kind not in ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm"):
+    if op.kind not in GEMM_KINDS:
         return [base]
     view = GemmView(op)
     i8 = view.dtype == "int8"

@@ -15,6 +15,9 @@
 //                             Grouped convolution (CG groups) runs one GEMM
 //                             per group: M = Kout/CG, K = (C/CG)*R*S, and the
 //                             group index is one more grid factor.
+//                             COLOUT 1 stores C as [CG][M][N], the layout of the
+//                             GEMM stage of a convolution written as im2col,
+//                             GEMM, col2img (ops.py:982-1044), instead of NCHW.
 //
 // Knobs (set by the scheduler from a Config):
 //   MFMA            32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
@@ -95,6 +98,11 @@
 #define DTL FT_DTL
 #else
 #define DTL 0
+#endif
+#ifdef FT_COLOUT
+#define COLOUT FT_COLOUT
+#else
+#define COLOUT 0
 #endif
 #ifdef FT_SK_PER
 #define SK_PER FT_SK_PER
@@ -369,7 +377,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
             for (int j = 0; j < REP_N; ++j) {
                 const int n = n0_ + (wn * REP_N + j) * MFMA + li;
-#if MODE == 1
+#if MODE == 1 && !COLOUT
                 const int b = n / OHW;
                 const int p = n % OHW;
                 const size_t cbase = ((size_t)b * (CG * M) + (size_t)gi_ * M) * OHW + p;
@@ -386,7 +394,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                     if (M % BM != 0) ok = ok && (m < M);
                     if (N % BN != 0) ok = ok && (n < N);
                     if (ok) {
-#if MODE == 1
+#if MODE == 1 && !COLOUT
                         float* dst = C + cbase + (size_t)m * OHW;
 #else
                         float* dst = C + ((size_t)gi_ * M + m) * N + n;

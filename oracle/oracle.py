@@ -191,6 +191,55 @@ def bias_add_nchw_np(y, bias):
     return (np.asarray(y, np.float32) + np.asarray(bias, np.float32)[None, :, None, None]).astype(np.float32)
 
 
+def im2col_nchw_np(x, kernel_shape, stride=1, padding=0, dilation=1, groups=1):
+    """col[g, h, w] gathered with the index expression of flextensor/nn/ops.py:943-949
+    (index arrays built from the formula itself; fp32 values are copied, not computed)."""
+    x = np.asarray(x, np.float32)
+    nb, c, h, w = x.shape
+    _, cg, r, s = [int(v) for v in kernel_shape]
+    p = conv_out_size(h, padding, dilation, r, stride)
+    q = conv_out_size(w, padding, dilation, s, stride)
+    xp = np.pad(x, ((0, 0), (0, 0), (padding, padding), (padding, padding)))
+    gi = np.arange(groups)[:, None, None]
+    hi = np.arange(cg * r * s)[None, :, None]
+    wi = np.arange(nb * p * q)[None, None, :]
+    return xp[wi // (p * q),
+              gi * cg + hi // (r * s),
+              wi % (p * q) // q * stride + hi % (r * s) // s * dilation,
+              wi % q * stride + hi % s * dilation]
+
+
+def col2img_nchw_np(y, p, q):
+    """O[b, c, h, w] = I[c // Mg, c % Mg, b*(P*Q) + h*Q + w] (flextensor/nn/ops.py:972-978)."""
+    y = np.asarray(y)
+    g, mg, width = y.shape
+    nb = width // (p * q)
+    bi = np.arange(nb)[:, None, None, None]
+    ci = np.arange(g * mg)[None, :, None, None]
+    hi = np.arange(p)[None, None, :, None]
+    wi = np.arange(q)[None, None, None, :]
+    return y[ci // mg, ci % mg, bi * (p * q) + hi * q + wi]
+
+
+def gemm_conv2d_nchw_np(x, wt, bias=None, stride=1, padding=0, dilation=1, groups=1):
+    """im2col, one float64 GEMM per group, optional bias, col2img
+    (flextensor/nn/ops.py:982-1044). Returns (output, col, gemm stage)."""
+    wt = np.asarray(wt, np.float32)
+    ko, cg, r, s = wt.shape
+    mg = ko // groups
+    col = im2col_nchw_np(x, wt.shape, stride, padding, dilation, groups)
+    ki = np.arange(cg * r * s)
+    # W[g*Mg + h, k // (kh*kw), k % (kh*kw) // kw, k % kw]
+    wmat = wt[:, ki // (r * s), ki % (r * s) // s, ki % s].reshape(groups, mg, cg * r * s)
+    gemm = np.einsum("ghk,gkw->ghw", wmat.astype(np.float64), col.astype(np.float64))
+    if bias is not None:
+        gemm = gemm + np.asarray(bias, np.float64).reshape(groups, mg, 1)
+    h, w = np.asarray(x).shape[2:]
+    p = conv_out_size(h, padding, dilation, r, stride)
+    q = conv_out_size(w, padding, dilation, s, stride)
+    return col2img_nchw_np(gemm, p, q), col, gemm
+
+
 def depthwise_nchw_np(x, wt, stride=1, padding=0, dilation=1):
     x = np.asarray(x, dtype=np.float64)
     wt = np.asarray(wt, dtype=np.float64)

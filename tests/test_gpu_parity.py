@@ -357,6 +357,84 @@ def test_conv2d_with_bias(oracle, args, kn, pad):
     assert rel(out.cpu().numpy(), ref) <= TOL
 
 
+def _gemm_conv_bias(N, C, H, W, K, k, stride=1, padding=0, dilation=1, groups=1):
+    from flextensor_amd.nn import gemm_conv2d_nchw
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((K, C // groups, k, k), name="W")
+    bias = placeholder((K,), name="bias")
+    Out = gemm_conv2d_nchw(Img, Wt, bias, stride=stride, padding=padding, dilation=dilation, groups=groups)
+    return [Out.op], [Img, Wt, bias, Out]
+
+
+@pytest.mark.parametrize("args,kn,pad,with_bias", [
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=16), [4, -1], False),
+    ((1, 384, 27, 27, 64, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, st=3), [-1, -1], True),   # the reference's test case
+    ((4, 6, 11, 9, 9, 3, 2, 1, 2, 3), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16), [4, -1], True),            # groups, stride, dilation, K tail
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=5, ks=1), [0, 0], False),   # straight into LDS, K streaming
+])
+def test_gemm_conv2d_vs_oracle(oracle, args, kn, pad, with_bias):
+    """[Padding, Img2Col, ComputeGemm, (ComputeBias,) Col2Img] under every
+    combination of graph flags that has a kernel sequence: from one implicit
+    GEMM kernel to pad, im2col, batched GEMM, bias, col2img as five kernels;
+    intermediates are checked through the final result."""
+    from flextensor_amd.task import gemm_conv2d
+    from flextensor_amd.templates.gfx950 import InvalidConfig
+    func = _gemm_conv_bias if with_bias else gemm_conv2d
+    register(func, "gemm_conv2d", "t", args, "rocm", 0, override=True)
+    key = key_of("gemm_conv2d", "t", args)
+    TASK_TABLE[key].set_specific_space("lds_pad", "enum", [pad])
+    ops, bufs = TASK_TABLE[key].func(*args)
+    host = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    x, w = host[0], host[1]
+    bias = host[2] if with_bias else None
+    ref = oracle.gemm_conv2d_nchw_np(x, w, bias, st, pd, dl, g)[0]
+    direct = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
+    if with_bias:
+        direct = oracle.bias_add_nchw_np(direct, bias)
+    assert rel(direct, ref) <= 1e-6
+    M, N, K = ko // g, nb * ref.shape[2] * ref.shape[3], (c // g) * ks * ks
+    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    cfg = gcfg(M, N, kp, **kn)
+    nops = 5 if with_bias else 4
+    empty = {k: [] for k in KEYS}
+    op_cfgs = [dict(empty), dict(empty), cfg] + [dict(empty)] * (nops - 3)
+    ran = 0
+    for pad_in in (1, 0):
+        for col_in in (1, 0):
+            for bias_m in ((1, 0) if with_bias else (0,)):
+                for img_m in (1, 0):
+                    gc = {k: [] for k in KEYS}
+                    gc["inline"] = [[pad_in, col_in] + [0] * (nops - 2)]
+                    gc["merge"] = [[0, 0, 0] + ([bias_m] if with_bias else []) + [img_m]]
+                    gc["special"] = [pad]
+                    configs = Config(op_cfgs, gc)
+                    try:
+                        plan, _ = schedule_with_config(key, configs)
+                    except InvalidConfig:
+                        # col2img merges only into the GEMM that reads the image, and only behind a merged bias
+                        assert img_m == 1 and (col_in == 0 or (with_bias and bias_m == 0)), gc
+                        continue
+                    kernels = [k_.kernel for k_ in plan.specs]
+                    assert ("zero_pad2d_f32" in kernels) == (pad_in == 0)
+                    assert ("im2col_nchw_f32" in kernels) == (col_in == 0)
+                    assert ("col2img_nchw_f32" in kernels) == (img_m == 0)
+                    if with_bias:
+                        assert ("bias_add_nchw_f32" in kernels) == (bias_m == 0)
+                    out = run_plan(key, configs, list(host))
+                    assert rel(out, ref) <= TOL, (gc["inline"], gc["merge"], kernels)
+                    ran += 1
+    assert ran == (10 if with_bias else 6)
+    # untuned replay and the default-schedule reference of the correctness gate
+    out = run_plan(key, Config([], None), list(host))
+    assert rel(out, ref) <= TOL
+    dev = [torch.from_numpy(a).cuda() for a in host]
+    out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+    run_default_schedule(ops, dev + [out], stream=current_stream())
+    torch.cuda.synchronize()
+    assert rel(out.cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("args,kn,pad", [
     ((5, 96, 80, 67), dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=16), [4, -1]),                  # ragged, scalar B loads
     ((3, 200, 136, 328), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=3), [-1, -1]),

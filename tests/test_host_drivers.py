@@ -6,7 +6,8 @@ import os
 
 import numpy as np
 
-from flextensor_amd.optimize import common, optimize_conv2d, optimize_depthwise_conv2d, optimize_gemm
+from flextensor_amd.optimize import (common, optimize_conv2d, optimize_depthwise_conv2d, optimize_gemm,
+                                     optimize_gemm_conv2d)
 from flextensor_amd.scheduler import schedule_with_config
 from flextensor_amd.task import TASK_TABLE
 from flextensor_amd.tuned import load, lookup
@@ -43,6 +44,11 @@ def test_driver_keys_are_registered():
             assert mk(i, shp, a)[0].key in TASK_TABLE, (table, i)
     mk = optimize_conv2d.make_task_for("yolo")
     assert mk(3, optimize_conv2d.SHAPES["yolo"][3], a)[0].key in TASK_TABLE
+    for table in ("yolo", "yolo_b8", "baseline"):
+        mk = optimize_gemm_conv2d.make_task_for(table)
+        for i, shp in enumerate(optimize_gemm_conv2d.SHAPES[table]):
+            task, trials = mk(i, shp, a)
+            assert task.key in TASK_TABLE and task.key.startswith("gemm_conv2d_") and len(trials) == 4
     for i, s in enumerate(optimize_depthwise_conv2d.SHAPES["baseline"] + optimize_depthwise_conv2d.SHAPES["mobile"]):
         assert optimize_depthwise_conv2d.make_task(i, s, a)[0].key in TASK_TABLE
 
@@ -83,3 +89,18 @@ def test_shipped_tuned_log_replays_for_every_benchmark_task():
         s, bufs = schedule_with_config(key, cfg)
         assert s.specs and len(bufs) == 3
     assert os.path.exists(os.path.join(os.path.dirname(common.__file__), "..", "tuned", "mi355x.log"))
+
+
+def test_tuned_convolution_points_carry_over_to_the_im2col_form():
+    """A gemm_conv2d task without an entry of its own replays the direct
+    convolution's tuned point: same kernel, same constants, no intermediates."""
+    key = "gemm_conv2d_yolo5_(1, 256, 56, 56, 512, 3, 1, 1, 1, 1)_rocm(0)"
+    direct = "conv2d_yolo5_(1, 256, 56, 56, 512, 3, 1, 1, 1, 1)_rocm(0)"
+    assert key not in load() and direct in load()
+    cfg = lookup(key)
+    assert len(cfg.op_config_lst) == 4 and cfg.op_config_lst[2] == lookup(direct).op_config_lst[1]
+    assert cfg.graph_config["inline"] == [[1, 1, 0, 0]] and cfg.graph_config["merge"] == [[0, 0, 0, 1]]
+    s, _ = schedule_with_config(key, cfg)
+    d, _ = schedule_with_config(direct, lookup(direct))
+    assert [k.defines for k in s.specs] == [k.defines for k in d.specs] and not s.intermediates
+    assert lookup("gemm_conv2d_nothing_(1,)_rocm(0)") is None

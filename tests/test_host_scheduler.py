@@ -192,6 +192,58 @@ def test_bias_stage_merges_into_the_convolution_or_runs_alone():
     assert [x.kernel for x in s.specs] == ["igemm_f32"]
 
 
+def test_gemm_conv2d_graph_flags_choose_the_kernel_sequence():
+    """Graph [Padding, Img2Col, ComputeGemm, Col2Img] (flextensor/nn/ops.py:982-1044):
+    inline and merge flags decide which stages exist as kernels; with everything
+    folded the plan is the direct convolution's kernel."""
+    from flextensor_amd.space import generate_space_inter_op
+    key = Task("gemm_conv2d", "yolo5", None, (1, 256, 56, 56, 512, 3, 1, 1, 1, 1), "rocm", 0).key
+    conv_key = Task("conv2d", "yolo5", None, (1, 256, 56, 56, 512, 3, 1, 1, 1, 1), "rocm", 0).key
+    task = TASK_TABLE[key]
+    ops, bufs = task.func(*task.args)
+    op_lst, down = flatten_graph(ops)
+    assert [(o.name, o.kind) for o in op_lst] == [("Padding", "zero_pad2d"), ("Img2Col", "im2col_nchw"),
+                                                   ("ComputeGemm", "col_gemm"), ("Col2Img", "col2img_nchw")]
+    assert op_lst[1].output(0).shape == (1, 2304, 3136) and op_lst[2].output(0).shape == (1, 512, 3136)
+    assert bufs[-1].shape == (1, 512, 56, 56)
+    gs = generate_space_inter_op(op_lst, down, special_space=task.special_space)
+    assert sorted(gs.subspaces["inline"].static_entities) == [[0, 0, 0, 0], [0, 1, 0, 0], [1, 0, 0, 0], [1, 1, 0, 0]]
+    assert sorted(gs.subspaces["merge"].static_entities) == [[0, 0, 0, 0], [0, 0, 0, 1]]
+    # defaults: one implicit-GEMM kernel, the same source and constants as conv2d's
+    s, _ = schedule_with_config(key, Config([], None))
+    c, _ = schedule_with_config(conv_key, Config([], None))
+    assert [x.kernel for x in s.specs] == ["igemm_f32"] and not s.intermediates
+    assert s.specs[0].defines == c.specs[0].defines and s.specs[0].grid == c.specs[0].grid
+
+    def plan(inline, merge):
+        g = {k: [] for k in ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]}
+        g["inline"], g["merge"] = [inline], [merge]
+        return schedule_with_config(key, Config([], g))[0]
+
+    s = plan([1, 1, 0, 0], [0, 0, 0, 0])
+    assert [x.kernel for x in s.specs] == ["igemm_f32", "col2img_nchw_f32"]
+    assert s.specs[0].defines["COLOUT"] == 1 and s.intermediates == {"tmp2": ((1, 512, 3136), "float32")}
+    s = plan([0, 0, 0, 0], [0, 0, 0, 0])
+    assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "im2col_nchw_f32", "igemm_f32", "col2img_nchw_f32"]
+    assert s.specs[1].defines["CH"] == 58 and s.specs[1].defines["CPAD"] == 0      # reads the padded image
+    assert s.specs[2].defines["MODE"] == 0 and [a[1] for a in s.specs[2].args] == ["in1", "tmp1", "tmp2"]
+    s = plan([1, 0, 0, 0], [0, 0, 0, 0])
+    assert s.specs[0].kernel == "im2col_nchw_f32" and s.specs[0].defines["CH"] == 56 and s.specs[0].defines["CPAD"] == 1
+    s = plan([0, 1, 0, 0], [0, 0, 0, 1])
+    assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "igemm_f32"]
+    assert s.specs[1].defines["CPAD"] == 0 and s.specs[1].defines["CH"] == 58 and "COLOUT" not in s.specs[1].defines
+    # the NCHW store belongs to the kernel that knows the image geometry
+    with pytest.raises(gfx950.InvalidConfig):
+        plan([1, 0, 0, 0], [0, 0, 0, 1])
+    # searched like any other task (host cost: fewer kernels is cheaper)
+    np.random.seed(3)
+    s, _, configs = schedule(key, op_trial=2, graph_trial=3, parallel=2, warm_up=(1, 4), verbose=False,
+                             trials=[1, 1, 2, 1],
+                             evaluator=lambda k, c, p, n: 1.0 + len(schedule_with_config(k, c, op_pos=p)[0].specs))
+    assert len(configs.op_config_lst) == 4 and [x.kernel for x in s.specs] == ["igemm_f32"]
+    assert configs.graph_config["inline"][0] == [1, 1, 0, 0] and configs.graph_config["merge"][0] == [0, 0, 0, 1]
+
+
 def test_batch_gemm_lowers_to_one_launch_over_all_matrices():
     from flextensor_amd.task import register, batch_gemm
     args = (6, 128, 96, 192)

@@ -104,6 +104,43 @@ def test_conv2d_bias_vs_torch(oracle):
     assert np.array_equal(z, np.broadcast_to(bias[None, :, None, None], z.shape))
 
 
+def test_gemm_conv2d_vs_torch_and_direct(oracle):
+    """im2col, GEMM, bias, col2img against torch's convolution, the check the
+    reference runs (flextensor/test/test_ops.py:254-284, 1x1 case with bias),
+    plus padded, strided, dilated and grouped cases and the intermediate
+    tensors against forms that share no indexing with the restatement."""
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    rng = np.random.default_rng(11)
+    for (n, c, h, w, k, r, st, p, d, g) in [
+            (1, 384, 27, 27, 64, 1, 1, 0, 1, 1),   # the reference's case
+            (2, 6, 9, 8, 4, 3, 1, 1, 1, 1),
+            (2, 6, 11, 9, 9, 3, 2, 1, 2, 3),
+            (1, 4, 7, 7, 6, 5, 1, 2, 1, 2)]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (k, c // g, r, r)).astype(np.float32)
+        bias = rng.uniform(-1, 1, (k,)).astype(np.float32)
+        ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(),
+                       torch.from_numpy(bias).double(), st, p, d, g).numpy()
+        out, col, stage = oracle.gemm_conv2d_nchw_np(x, wt, bias, st, p, d, g)
+        assert out.shape == ref.shape
+        assert rel(out, ref) < 1e-12
+        # without bias it is the direct convolution's own restatement
+        assert rel(oracle.gemm_conv2d_nchw_np(x, wt, None, st, p, d, g)[0],
+                   oracle.conv2d_nchw_c(x, wt, st, p, d, g)) < 1e-6
+        # the column matrix is torch's unfold, group by group
+        unf = F.unfold(torch.from_numpy(x), r, dilation=d, padding=p, stride=st).numpy()   # [n, c*r*r, P*Q]
+        pq = unf.shape[2]
+        cg = c // g
+        for gi in range(g):
+            want = unf[:, gi * cg * r * r:(gi + 1) * cg * r * r].transpose(1, 0, 2).reshape(cg * r * r, n * pq)
+            assert np.array_equal(col[gi], want)
+        # col2img is a pure permutation: [g, Mg, n, P*Q] -> [n, g*Mg, P, Q]
+        mg = k // g
+        want = stage.reshape(g * mg, n, pq).transpose(1, 0, 2).reshape(ref.shape)
+        assert np.array_equal(out, want)
+
+
 def test_conv2d_linearity_and_delta(oracle):
     rng = np.random.default_rng(2)
     x1 = rng.uniform(-1, 1, (1, 3, 6, 6)).astype(np.float32)

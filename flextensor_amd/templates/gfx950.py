@@ -696,9 +696,11 @@ def seed_configs(op, limit=24):
         bks, depths, streams = [128, 64], [7, 6, 2], [0]
     else:
         shapes = [((4, 1, 16), (4, 1, 16)), ((4, 1, 32), (2, 1, 32)), ((2, 1, 32), (2, 1, 32)),
-                  ((4, 1, 16), (1, 1, 16)), ((4, 1, 16), (2, 1, 16)), ((2, 2, 16), (4, 1, 16))]
+                  ((4, 1, 16), (1, 1, 16)), ((4, 1, 16), (2, 1, 16)), ((2, 2, 16), (4, 1, 16)),
+                  ((2, 1, 16), (4, 1, 16))]
         bks = [b for b in (144, 72, 64, 48, 32) if b in F32_BK]
         depths, streams = [5, 3, 2, 1], [0, 1]
+    split_seeds = []
     for (m_w, m_r, mf), (n_w, n_r, _) in shapes:
         tm, tn = tile(view.M, m_w, m_r, mf), tile(view.N, n_w, n_r, mf)
         tiles = tm[0] * tn[0] * view.groups
@@ -717,8 +719,26 @@ def seed_configs(op, limit=24):
                     cfg["fuse"] = [[8]]
                     cfg["reorder"] = [[1, 0, stream]]
                     out.append(cfg)
+                if not i8 and depth == depths[0] and tiles * 2 <= NUM_CUS:
+                    # few tiles and a long K (weights streamed past a small image): K parts across
+                    # workgroups, as many as fill the compute units
+                    split = 1
+                    while split * 2 * tiles <= NUM_CUS and split < 16 and (kps[0] // bk) % (split * 2) == 0:
+                        split *= 2
+                    if split > 1:
+                        cfg = _empty_config()
+                        cfg["spatial"] = [tm, tn]
+                        cfg["reduce"] = [[split, kps[0] // (bk * split), bk]]
+                        cfg["unroll"] = [[depth, 1]]
+                        cfg["fuse"] = [[8]]
+                        cfg["reorder"] = [[1, 0, 0]]
+                        split_seeds.append(cfg)
     # spread over the variations instead of exhausting the first tile shape
-    if len(out) > limit:
-        step = (len(out) - 1) / float(limit - 1)
-        out = [out[int(round(i * step))] for i in range(limit)]
-    return out
+    def spread(lst, n):
+        if len(lst) <= n:
+            return lst
+        step = (len(lst) - 1) / float(max(n - 1, 1))
+        return [lst[int(round(i * step))] for i in range(n)]
+
+    nsplit = min(len(split_seeds), limit // 3)
+    return spread(out, limit - nsplit) + spread(split_seeds, nsplit)

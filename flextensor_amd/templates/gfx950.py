@@ -284,7 +284,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         raise InvalidConfig("only the convolution has a bias epilogue")
     if merged_out is not None and not (op.kind == "col_gemm" and merged_out == "col2img_nchw"):
         raise InvalidConfig("stage %s cannot run in the stores of %s" % (merged_out, op.kind))
-    if merged_out is not None and view.mode != 1:
+    if merged_out is not None and view.mode != 1 and view.conv["CB"] != 1:
+        # for one image [groups][M][P*Q] is NCHW already; a batch interleaves the images
         raise InvalidConfig("col2img merges into the GEMM that reads the image itself")
     sp = _one(config, "spatial", 2, op.kind)
     rd = _one(config, "reduce", 1, op.kind)

@@ -371,6 +371,7 @@ def _gemm_conv_bias(N, C, H, W, K, k, stride=1, padding=0, dilation=1, groups=1)
     ((1, 384, 27, 27, 64, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, st=3), [-1, -1], True),   # the reference's test case
     ((4, 6, 11, 9, 9, 3, 2, 1, 2, 3), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16), [4, -1], True),            # groups, stride, dilation, K tail
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=5, ks=1), [0, 0], False),   # straight into LDS, K streaming
+    ((1, 16, 14, 14, 48, 3, 1, 1, 1, 2), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=8, sk=3, st=3), [4, -1], False),  # one image, groups, split K
 ])
 def test_gemm_conv2d_vs_oracle(oracle, args, kn, pad, with_bias):
     """[Padding, Img2Col, ComputeGemm, (ComputeBias,) Col2Img] under every
@@ -412,8 +413,9 @@ def test_gemm_conv2d_vs_oracle(oracle, args, kn, pad, with_bias):
                     try:
                         plan, _ = schedule_with_config(key, configs)
                     except InvalidConfig:
-                        # col2img merges only into the GEMM that reads the image, and only behind a merged bias
-                        assert img_m == 1 and (col_in == 0 or (with_bias and bias_m == 0)), gc
+                        # col2img merges only behind a merged bias, and into the GEMM over stored
+                        # columns only for one image (where [groups][M][P*Q] is NCHW already)
+                        assert img_m == 1 and ((col_in == 0 and nb > 1) or (with_bias and bias_m == 0)), gc
                         continue
                     kernels = [k_.kernel for k_ in plan.specs]
                     assert ("zero_pad2d_f32" in kernels) == (pad_in == 0)
@@ -424,7 +426,7 @@ def test_gemm_conv2d_vs_oracle(oracle, args, kn, pad, with_bias):
                     out = run_plan(key, configs, list(host))
                     assert rel(out, ref) <= TOL, (gc["inline"], gc["merge"], kernels)
                     ran += 1
-    assert ran == (10 if with_bias else 6)
+    assert ran == (10 if with_bias else 6) + ((2 if with_bias else 2) if nb == 1 else 0)
     # untuned replay and the default-schedule reference of the correctness gate
     out = run_plan(key, Config([], None), list(host))
     assert rel(out, ref) <= TOL

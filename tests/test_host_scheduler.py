@@ -232,9 +232,15 @@ def test_gemm_conv2d_graph_flags_choose_the_kernel_sequence():
     s = plan([0, 1, 0, 0], [0, 0, 0, 1])
     assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "igemm_f32"]
     assert s.specs[1].defines["CPAD"] == 0 and s.specs[1].defines["CH"] == 58 and "COLOUT" not in s.specs[1].defines
-    # the NCHW store belongs to the kernel that knows the image geometry
+    # one image: [groups][M][P*Q] is NCHW already, so the GEMM over stored columns writes the output itself
+    s = plan([1, 0, 0, 0], [0, 0, 0, 1])
+    assert [x.kernel for x in s.specs] == ["im2col_nchw_f32", "igemm_f32"] and s.specs[1].args[2] == ("buf", "out")
+    # a batch interleaves the images: then the NCHW store belongs to the kernel that knows the geometry
+    key8 = Task("gemm_conv2d", "yolo_b85", None, (8, 256, 56, 56, 512, 3, 1, 1, 1, 1), "rocm", 0).key
+    g8 = {k: [] for k in ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]}
+    g8["inline"], g8["merge"] = [[1, 0, 0, 0]], [[0, 0, 0, 1]]
     with pytest.raises(gfx950.InvalidConfig):
-        plan([1, 0, 0, 0], [0, 0, 0, 1])
+        schedule_with_config(key8, Config([], g8))
     # searched like any other task (host cost: fewer kernels is cheaper)
     np.random.seed(3)
     s, _, configs = schedule(key, op_trial=2, graph_trial=3, parallel=2, warm_up=(1, 4), verbose=False,

@@ -194,7 +194,7 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7] if i8 else [1, 2, 3, 4, 5], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7], explicit=True), "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
     space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
@@ -244,7 +244,8 @@ SPECIAL_DEFAULTS = {
 # depth 5 = two stages with the fragment-prefetch pipeline (int8 GEMM)
 # depth -> (LDS buffers, global prefetch distance); 5 = int8: MFMA fragment prefetch, fp32: tiles
 # loaded straight into LDS; int8 only:
-# 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch
+# 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch;
+# fp32: 6 and 7 = 5 with three and four LDS buffers (two and three tiles requested ahead)
 PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7: (2, 1)}
 
 
@@ -292,9 +293,11 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE or (depth >= 6 and view.dtype != "int8"):
+    if depth not in PIPELINE:
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
+    if view.dtype != "int8" and depth >= 6:
+        stages = depth - 3        # fp32: 6 and 7 = tiles straight into LDS with three and four buffers
     group_m = int((config.get("fuse") or [[4]])[0][0])
     ro = list((config.get("reorder") or [[1, 0]])[0]) + [0, 0]
     xcd, in_wg, stream_k = int(ro[0]), int(ro[1]), int(ro[2])
@@ -377,7 +380,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         bv = av
     else:
         bv = 1
-    dtl = depth == 5          # fp32: tiles loaded straight into LDS
+    dtl = depth >= 5          # fp32: tiles loaded straight into LDS
     if dtl:
         if view.mode == 0 and view.N % 4 == 0 and bn % 64 == 0 and (bpad_auto or bpad == 0):
             bv, bpad = 4, 0   # B in 16-byte chunks too: unpadded rows, columns swizzled by k
@@ -408,6 +411,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     eb = ceil_div((bn * bk) // bv, nt)
     if not dtl and (ea * av + eb * bv) * pd > 160:
         raise InvalidConfig("global->LDS staging needs too many registers")
+    if dtl and stages > 2 and ((bm * bk // av) % nt or ((bn * bk) // bv) % nt or (stages - 2) * (ea + eb) > 63):
+        raise InvalidConfig("more than two direct-to-LDS buffers need whole rounds of loads per tile, "
+                            "at most 63 of them in flight")
     if max(view.M * view.K, view.K * view.N, view.M * view.N) * view.groups * 4 >= 2 ** 31:
         raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
     D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)

@@ -24,7 +24,7 @@
 //   WAVES_M/N       wavefronts per workgroup along M / N
 //   REP_M/N         MFMA tiles per wavefront along M / N
 //   BK              K extent of one LDS tile
-//   STAGES          1 or 2 LDS buffers (2 = the LDS stores of tile t+1 need no
+//   STAGES          1 or 2 LDS buffers, 3 or 4 with DTL (2 = the LDS stores of tile t+1 need no
 //                   extra barrier against the reads of tile t)
 //   PD              prefetch distance: global loads of tile t+PD are in
 //                   flight (in PD register sets) while tile t is multiplied
@@ -188,9 +188,15 @@ typedef f32x4 acc_t;
 #endif
 #define EB ((B_CHUNKS + NT - 1) / NT)
 #if DTL
-#if STAGES != 2 || PD != 1 || AV != 4 || APAD > 0 || A_CHUNKS % 64 != 0 || B_CHUNKS % 64 != 0
-#error "direct-to-LDS tiles: two buffers, 16-byte A chunks, unpadded A rows, whole wavefronts of chunks"
+#if STAGES < 2 || STAGES > 4 || PD != 1 || AV != 4 || APAD > 0 || A_CHUNKS % 64 != 0 || B_CHUNKS % 64 != 0
+#error "direct-to-LDS tiles: two to four buffers, 16-byte A chunks, unpadded A rows, whole wavefronts of chunks"
 #endif
+#if STAGES > 2 && (A_CHUNKS % NT != 0 || B_CHUNKS % NT != 0 || (STAGES - 2) * (EA + EB) > 63)
+#error "more than two direct-to-LDS buffers: every wavefront must issue the same number of loads per tile"
+#endif
+/* loads one wavefront issues per tile, and a wait that lets the newest n loads stay in flight */
+#define DMA_PER_TILE (EA + EB)
+#define VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #if MODE == 2
 #if BV != 4
 #error "direct-to-LDS tiles: B^T needs 16-byte chunks"
@@ -771,7 +777,32 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         arrive_tile = -1;
     }
 #endif
-#if DTL
+#if DTL && STAGES > 2
+    /* STAGES buffers: tiles 1 .. STAGES-2 are requested right behind tile 0,
+     * and tile kt+STAGES-1 while tile kt is multiplied, so STAGES-1 tiles are
+     * in flight or landed ahead of the MFMAs. Loads complete in order: a wait
+     * that leaves the loads of the tiles behind kt+1 outstanding has seen
+     * tile kt+1 land. */
+#pragma unroll
+    for (int p = 1; p < STAGES - 1; ++p)
+        if (p < nk) dma_tile(p, p);
+    {
+        int cur = 0, nxt = STAGES - 1;       /* buffers of tile kt and of tile kt+STAGES-1 */
+        for (int kt = 0; kt < nk; ++kt) {
+            if (kt + STAGES - 1 < nk) dma_tile(kt + STAGES - 1, nxt);
+            compute(cur);
+            const int behind = nk - kt - 2;  /* requested tiles behind tile kt+1 (more than STAGES-2 never are) */
+            if (behind >= STAGES - 2) VMCNT((STAGES - 2) * DMA_PER_TILE);
+#if STAGES > 3
+            else if (behind == 1) VMCNT(DMA_PER_TILE);
+#endif
+            else VMCNT(0);
+            __syncthreads();
+            cur = (cur + 1 == STAGES) ? 0 : cur + 1;
+            nxt = (nxt + 1 == STAGES) ? 0 : nxt + 1;
+        }
+    }
+#elif DTL
     for (int kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
         if (kt + 1 < nk) dma_tile(kt + 1, cur ^ 1);      /* lands while tile kt is multiplied */

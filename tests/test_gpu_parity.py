@@ -252,9 +252,16 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     (96, 144, 128, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=72, st=5), [0, 0]),               # partial last round of chunks
     (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=5), [0, 0]),               # B in swizzled 16-byte chunks, ragged
     (256, 256, 512, dict(wm=2, rm=2, wn=2, rn=4, mf=16, bk=32, st=5), [-1, -1]),            # same, 128-wide tile
+    # three and four buffers: two and three tiles requested ahead
+    (256, 512, 256, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=64, st=6), [-1, -1]),
+    (256, 512, 256, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=7), [-1, -1]),
+    (256, 64, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=7), [-1, -1]),             # fewer tiles than buffers
+    (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16, st=6), [0, 0]),               # ragged, padded K, odd tile count
+    (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=6, ks=1), [-1, -1]),      # with K streaming: segments of any length
+    (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=7, ks=2), [-1, -1]),
 ])
 def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
-    """Pipeline depth 5: tiles travel global -> LDS without staging registers."""
+    """Pipeline depths 5 to 7: tiles travel global -> LDS without staging registers."""
     register(gemm, "gemm", "gemm", (M, K, N), "rocm", 0)
     key = key_of("gemm", "gemm", (M, K, N))
     ops, bufs = TASK_TABLE[key].func(M, K, N)
@@ -297,6 +304,10 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     # accumulators right after the last MFMA (the store once came 19 issue slots too early)
     ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64, st=5, ks=1), [-1, 0]),
     ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=32, st=2, ks=1), [-1, 0]),
+    # three and four buffers
+    ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16, st=6), [-1, 8]),
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=72, st=6), [0, 0]),
+    ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=32, st=7, ks=1), [-1, 0]),
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)

@@ -33,6 +33,72 @@ _yolo_layers = [
 yolo_shapes = [_conv(1, c, hw, k, ks, st, pd) for (c, hw, k, ks, st, pd) in _yolo_layers]
 yolo_shapes_b8 = [_conv(8, c, hw, k, ks, st, pd) for (c, hw, k, ks, st, pd) in _yolo_layers]
 
+# The other networks of the reference's conv2d tables (configs/conv2d_config.py:9-16, 58-67,
+# 83-268), as (C, H=W, K, kernel, stride, pad[, groups]); batch as the reference registers them.
+_overfeat_layers = [
+    (3, 192, 96, 11, 4, 5), (96, 24, 256, 5, 1, 2), (256, 12, 512, 3, 1, 1),
+    (512, 12, 1024, 3, 1, 1), (1024, 12, 1024, 3, 1, 1),
+]
+_google_layers = [
+    (3, 224, 64, 7, 2, 3), (64, 56, 64, 1, 1, 0), (64, 56, 192, 3, 1, 1), (192, 28, 64, 1, 1, 0),
+    (192, 28, 96, 1, 1, 0), (96, 28, 128, 3, 1, 1), (192, 28, 16, 1, 1, 0), (16, 28, 32, 5, 1, 2),
+    (192, 28, 32, 1, 1, 0), (256, 28, 128, 1, 1, 0), (128, 28, 192, 3, 1, 1),
+    (256, 28, 32, 1, 1, 0), (32, 28, 96, 5, 1, 2), (256, 28, 64, 1, 1, 0), (480, 14, 192, 1, 1, 0),
+    (480, 14, 96, 1, 1, 0), (96, 14, 208, 3, 1, 1), (480, 14, 16, 1, 1, 0), (16, 14, 48, 5, 1, 2),
+    (480, 14, 64, 1, 1, 0), (512, 14, 160, 1, 1, 0), (512, 14, 112, 1, 1, 0),
+    (112, 14, 224, 3, 1, 1), (512, 14, 24, 1, 1, 0), (24, 14, 64, 5, 1, 2), (512, 14, 64, 1, 1, 0),
+    (512, 14, 128, 1, 1, 0), (128, 14, 256, 3, 1, 1), (512, 14, 144, 1, 1, 0),
+    (144, 14, 288, 3, 1, 1), (512, 14, 32, 1, 1, 0), (32, 14, 64, 5, 1, 2),
+    (528, 14, 256, 1, 1, 0), (528, 14, 160, 1, 1, 0), (160, 14, 320, 3, 1, 1),
+    (528, 14, 32, 1, 1, 0), (32, 14, 128, 5, 1, 2), (528, 14, 128, 1, 1, 0),
+    (832, 7, 256, 1, 1, 0), (832, 7, 160, 1, 1, 0), (160, 7, 320, 3, 1, 1), (832, 7, 32, 1, 1, 0),
+    (32, 7, 128, 5, 1, 2), (832, 7, 128, 1, 1, 0), (832, 7, 384, 1, 1, 0), (832, 7, 192, 1, 1, 0),
+    (192, 7, 384, 3, 1, 1), (832, 7, 48, 1, 1, 0), (48, 7, 128, 5, 1, 2),
+]
+_squeeze_layers = [
+    (3, 227, 96, 7, 2, 0), (96, 55, 16, 1, 1, 0), (16, 55, 64, 1, 1, 0), (16, 55, 64, 3, 1, 1),
+    (128, 55, 16, 1, 1, 0), (128, 55, 32, 1, 1, 0), (32, 55, 128, 1, 1, 0), (32, 55, 128, 3, 1, 1),
+    (256, 27, 32, 1, 1, 0), (32, 27, 128, 1, 1, 0), (32, 27, 128, 3, 1, 1), (256, 27, 48, 1, 1, 0),
+    (48, 27, 192, 1, 1, 0), (48, 27, 192, 3, 1, 1), (384, 27, 48, 1, 1, 0), (384, 27, 64, 1, 1, 0),
+    (64, 27, 256, 1, 1, 0), (64, 27, 256, 3, 1, 1), (512, 13, 64, 1, 1, 0), (64, 13, 256, 1, 1, 0),
+    (64, 13, 256, 3, 1, 1), (512, 13, 1000, 1, 1, 0),
+]
+_res_layers = [
+    (3, 224, 64, 7, 2, 3), (64, 56, 256, 1, 1, 0), (64, 56, 64, 1, 1, 0), (64, 56, 64, 3, 1, 1),
+    (256, 56, 64, 1, 1, 0), (256, 56, 512, 1, 2, 0), (256, 56, 128, 1, 2, 0),
+    (128, 28, 128, 3, 1, 1), (128, 28, 512, 1, 1, 0), (512, 28, 128, 1, 1, 0),
+    (512, 28, 1024, 1, 2, 0), (512, 28, 256, 1, 2, 0), (256, 14, 256, 3, 1, 1),
+    (256, 14, 1024, 1, 1, 0), (1024, 14, 256, 1, 1, 0), (1024, 14, 2048, 1, 2, 0),
+    (1024, 14, 512, 1, 2, 0), (512, 7, 512, 3, 1, 1), (512, 7, 2048, 1, 1, 0),
+    (2048, 7, 512, 1, 1, 0),
+]
+_vgg_16_layers = [
+    (3, 224, 64, 3, 1, 1), (64, 224, 64, 3, 1, 1), (64, 112, 128, 3, 1, 1),
+    (128, 112, 128, 3, 1, 1), (128, 56, 256, 3, 1, 1), (256, 56, 256, 3, 1, 1),
+    (256, 28, 512, 3, 1, 1), (512, 28, 512, 3, 1, 1), (512, 14, 512, 3, 1, 1),
+]
+# MobileNet-v2 depthwise stages written as grouped convolutions (groups = C)
+_mobilev2_layers = [
+    (32, 112, 32, 3, 1, 1, 32), (16, 112, 96, 3, 2, 1, 16), (24, 56, 144, 3, 2, 1, 24),
+    (32, 28, 192, 3, 2, 1, 32), (64, 14, 384, 3, 1, 1, 64), (96, 14, 576, 3, 2, 1, 96),
+    (160, 7, 960, 3, 1, 1, 160),
+]
+
+
+def _table(batch, layers):
+    return [_conv(batch, l[0], l[1], l[2], l[3], l[4], l[5], 1, l[6] if len(l) > 6 else 1) for l in layers]
+
+
+overfeat_shapes = _table(1, _overfeat_layers)
+google_shapes = _table(1, _google_layers)
+squeeze_shapes = _table(1, _squeeze_layers)
+res_shapes = _table(64, _res_layers)                 # the reference tunes ResNet at batch 64
+vgg_16_shapes = _table(1, _vgg_16_layers)
+vgg_19_shapes = []                                   # empty upstream as well (every entry commented out)
+mobilev2_shapes = _table(1, _mobilev2_layers)
+# one 1x1 layer at batch 256; its bias slot is 0 where the others carry 1 (never read by the drivers)
+test_conv_shapes = [(256, 256, 14, 14, 512, 256, 1, 1, 0, 1, 0, 1, 1)]
+
 # MobileNet-style depthwise layers
 depthwise_shapes = [
     (1, 32, 112, 112, 1, 3, 3, 1, 1, 1),

@@ -5,13 +5,13 @@ flextensor/optimize/optimize_conv2d.py:29-140 for the gfx950 backend.
 """
 import argparse
 
-from ..configs.shapes import (baseline_conv_shapes, yolo_shapes, yolo_shapes_b8, grouped_shapes,
-                              dilation_shapes)
-from ..task import Task
+from ..configs.shapes import grouped_shapes, dilation_shapes, vgg_19_shapes
+from ..task import Task, conv2d_shape_dict
 from .common import init_arg_parser, run_driver
 
-SHAPES = {"baseline": baseline_conv_shapes, "yolo": yolo_shapes, "yolo_b8": yolo_shapes_b8,
-          "grouped": grouped_shapes, "dilation": dilation_shapes}
+# the reference's tables (optimize_conv2d.py:17-26) plus the benchmark shapes and the two single-name tables
+SHAPES = dict(conv2d_shape_dict)
+SHAPES.update({"vgg-19": vgg_19_shapes, "grouped": grouped_shapes, "dilation": dilation_shapes})
 
 
 def make_task_for(prefix):

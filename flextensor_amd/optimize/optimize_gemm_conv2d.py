@@ -11,11 +11,13 @@ intermediate tensors the flags name.
 """
 import argparse
 
-from ..configs.shapes import baseline_conv_shapes, yolo_shapes, yolo_shapes_b8
-from ..task import Task
+from ..configs.shapes import vgg_19_shapes
+from ..task import Task, conv2d_shape_dict
 from .common import init_arg_parser, run_driver
 
-SHAPES = {"baseline": baseline_conv_shapes, "yolo": yolo_shapes, "yolo_b8": yolo_shapes_b8}
+# flextensor/optimize/optimize_gemm_conv2d.py:17-24 plus the benchmark shapes
+SHAPES = dict(conv2d_shape_dict)
+SHAPES["vgg-19"] = vgg_19_shapes
 
 
 def make_task_for(prefix):

@@ -13,7 +13,16 @@ from .space import EnumSpace
 from .te import placeholder
 from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8, grouped_shapes, dilation_shapes,
                              depthwise_shapes, baseline_conv_shapes, baseline_depthwise_shapes,
-                             baseline_gemm_shapes, baseline_gemm_int8_shapes)
+                             baseline_gemm_shapes, baseline_gemm_int8_shapes, google_shapes, res_shapes,
+                             squeeze_shapes, vgg_16_shapes, test_conv_shapes, mobilev2_shapes,
+                             overfeat_shapes)
+
+# table name -> conv2d shapes, the names of flextensor/task.py:274-284 plus this backend's benchmark shapes
+conv2d_shape_dict = {
+    "yolo": yolo_shapes, "google": google_shapes, "res": res_shapes, "squeeze": squeeze_shapes,
+    "vgg-16": vgg_16_shapes, "test": test_conv_shapes, "yolo_b8": yolo_shapes_b8,
+    "mobile_v2": mobilev2_shapes, "overfeat": overfeat_shapes, "baseline": baseline_conv_shapes,
+}
 
 TASK_TABLE = {}
 
@@ -132,8 +141,7 @@ def _register_all():
         for shape in baseline_gemm_int8_shapes:
             N, K, M = shape
             register(gemm_int8, "gemm", "gemm_int8", (N, K, M), ROCM_TARGET, j)
-        for name, shapes in (("yolo", yolo_shapes), ("yolo_b8", yolo_shapes_b8),
-                             ("baseline", baseline_conv_shapes)):
+        for name, shapes in conv2d_shape_dict.items():
             for i, shape in enumerate(shapes):
                 batch, in_c, h, w, out_c, _, k_h, k_w, _, stride, pad, dil, groups = shape
                 register(conv2d, "conv2d", name + str(i),

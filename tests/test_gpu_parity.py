@@ -758,15 +758,21 @@ def _registered_layer_keys():
     # yolo at batch 8 repeats the batch-1 layers with 8x the work: keep every third of them
     b8 = [k for k in keys if k.startswith("conv2d_yolo_b8")]
     keys = [k for k in keys if not k.startswith("conv2d_yolo_b8")] + b8[::3]
+    # the other networks' tables: every fourth layer of each (all of the short ones)
+    for prefix, step in (("conv2d_google", 4), ("conv2d_res", 4), ("conv2d_squeeze", 4), ("conv2d_vgg-16", 3),
+                         ("conv2d_overfeat", 2), ("conv2d_mobile_v2", 2)):
+        net = sorted(k for k in keys if k.startswith(prefix))
+        keys = [k for k in keys if not k.startswith(prefix)] + net[::step]
     return sorted(keys) + ["gemm_gemm_(32, 32, 32)_rocm(0)", "gemm_gemm_(4096, 32, 64)_rocm(0)",
                            "gemm_gemm_(64, 4096, 4096)_rocm(0)", "gemm_gemm_(2048, 2048, 2048)_rocm(0)"]
 
 
 @pytest.mark.parametrize("key", _registered_layer_keys())
 def test_registered_tasks_default_config_passes_the_gate(key):
-    """Every registered convolution layer (YOLO, grouped, dilated, depthwise,
-    the benchmark shapes) and a few GEMM shapes: the untuned plan matches the
-    default-schedule kernels on the device."""
+    """Registered convolution layers (all of YOLO, grouped, dilated, depthwise
+    and the benchmark shapes, a sample of the other networks' tables) and a
+    few GEMM shapes: the untuned plan matches the default-schedule kernels on
+    the device."""
     s, bufs = schedule_with_config(key, Config([], None))
     s.compile()                                   # from the on-disk cache when built ahead of time
     ms = Measurer(key).evaluate(s, number=3, warmup=1, warm_ms=0)

@@ -42,9 +42,17 @@ def test_driver_keys_are_registered():
         mk = optimize_conv2d.make_task_for(table)
         for i, shp in enumerate(optimize_conv2d.SHAPES[table]):
             assert mk(i, shp, a)[0].key in TASK_TABLE, (table, i)
-    mk = optimize_conv2d.make_task_for("yolo")
-    assert mk(3, optimize_conv2d.SHAPES["yolo"][3], a)[0].key in TASK_TABLE
-    for table in ("yolo", "yolo_b8", "baseline"):
+    # the reference's table names (optimize_conv2d.py:17-26), every layer registered for both conv forms
+    assert set(optimize_conv2d.SHAPES) >= {"yolo", "google", "squeeze", "res", "vgg-16", "vgg-19", "yolo_b8", "mobile_v2"}
+    assert [len(optimize_conv2d.SHAPES[n]) for n in ("yolo", "google", "squeeze", "res", "vgg-16", "vgg-19", "mobile_v2",
+                                                     "overfeat", "test")] == [15, 49, 22, 20, 9, 0, 7, 5, 1]
+    for table in ("yolo", "google", "squeeze", "res", "vgg-16", "mobile_v2", "overfeat", "test"):
+        mk, mk2 = optimize_conv2d.make_task_for(table), optimize_gemm_conv2d.make_task_for(table)
+        for i, shp in enumerate(optimize_conv2d.SHAPES[table]):
+            assert mk(i, shp, a)[0].key in TASK_TABLE and mk2(i, shp, a)[0].key in TASK_TABLE, (table, i)
+    assert "conv2d_res5_(64, 256, 56, 56, 512, 1, 2, 0, 1, 1)_rocm(0)" in TASK_TABLE
+    assert "conv2d_mobile_v21_(1, 16, 112, 112, 96, 3, 2, 1, 1, 16)_rocm(0)" in TASK_TABLE
+    for table in ("yolo_b8", "baseline"):
         mk = optimize_gemm_conv2d.make_task_for(table)
         for i, shp in enumerate(optimize_gemm_conv2d.SHAPES[table]):
             task, trials = mk(i, shp, a)

@@ -686,7 +686,9 @@ def seed_configs(op, limit=24):
     and variations of it along the knobs that decided the hand-tuned shapes
     (tile aspect and MFMA edge, LDS tile extent incl. whole 3x3 windows,
     pipeline depth incl. tiles straight into LDS, K streaming when the tiles
-    are fewer than the compute units). Only entities of the op's space are
+    are fewer than the compute units, and for layers with few tiles and a
+    long K a grid-level K split sized to fill the compute units; a third of
+    the points is kept for those). Only entities of the op's space are
     produced; points the templates refuse are dropped by the caller."""
     base = default_config(op)
     if op.kind not in GEMM_KINDS:

@@ -688,8 +688,10 @@ def seed_configs(op, limit=24):
     pipeline depth incl. tiles straight into LDS, K streaming when the tiles
     are fewer than the compute units, and for layers with few tiles and a
     long K a grid-level K split sized to fill the compute units; a third of
-    the points is kept for those). Only entities of the op's space are
-    produced; points the templates refuse are dropped by the caller."""
+    the points is kept for those). The variations are entities of the op's
+    space (the default config itself need not be: it may waste more of an
+    edge tile than the space admits); points the templates refuse are
+    dropped by the caller."""
     base = default_config(op)
     if op.kind not in GEMM_KINDS:
         return [base]
@@ -709,9 +711,18 @@ def seed_configs(op, limit=24):
                   ((2, 1, 16), (4, 1, 16))]
         bks = [b for b in (144, 72, 64, 48, 32) if b in F32_BK]
         depths, streams = [5, 3, 2, 1], [0, 1]
+    def in_space(extent, t):
+        # the tile space's own rules: no tile a smaller one covers as well, bounded edge waste
+        size = t[1] * t[2] * t[3]
+        if t[0] == 1:
+            return size - extent < t[3]
+        return t[0] * size - extent <= 0.25 * extent
+
     split_seeds = []
     for (m_w, m_r, mf), (n_w, n_r, _) in shapes:
         tm, tn = tile(view.M, m_w, m_r, mf), tile(view.N, n_w, n_r, mf)
+        if not (in_space(view.M, tm) and in_space(view.N, tn)):
+            continue
         tiles = tm[0] * tn[0] * view.groups
         for bk in bks:
             kps = [kp for kp in view.KP_options if kp % bk == 0]

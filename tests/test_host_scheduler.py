@@ -388,3 +388,36 @@ def test_walker_group_heap_semantics():
     # a hopeless value is (almost surely) rejected by the Boltzmann filter
     wg.record(nxt[0], 1e9, random_reject=True)
     assert wg.mem_size == 4 and wg.ever_met(nxt[0])
+
+
+def test_seed_points_cover_the_decisive_knobs_and_belong_to_the_space():
+    """The heuristic points measured before the random warm-up: inside the
+    operator's space, bounded in number, with direct-to-LDS depths, whole 3x3
+    windows, K streaming for few tiles, and grid-level K splits for layers
+    whose weights stream past a small image."""
+    def seeds_of(key):
+        task = TASK_TABLE[key]
+        ops, _ = task.func(*task.args)
+        op_lst, down = flatten_graph(ops)
+        op = [o for o in op_lst if o.kind in gfx950.GEMM_KINDS][0]
+        return op, generate_space_intra_op(op, down, target="rocm"), gfx950.seed_configs(op)
+
+    for key in (GEMM, CONV, CONV1x1, I8, "conv2d_yolo14_(1, 1024, 7, 7, 1024, 3, 1, 1, 1, 1)_rocm(0)"):
+        op, space, seeds = seeds_of(key)
+        assert 1 <= len(seeds) <= 24, key
+        assert seeds[0] == gfx950.default_config(op)
+        for cfg in seeds[1:]:
+            # every knob value of the variations is an entity of its sub-space
+            assert space.subspaces["split_m_0"].index_of(cfg["spatial"][0]) >= 0, (key, cfg["spatial"])
+            assert space.subspaces["split_n_1"].index_of(cfg["spatial"][1]) >= 0, (key, cfg["spatial"])
+            assert space.subspaces["split_k_0"].index_of(cfg["reduce"][0]) >= 0, (key, cfg["reduce"])
+    _, _, seeds = seeds_of(CONV)
+    assert any(c["unroll"][0][0] == 5 for c in seeds) and any(c["reduce"][0][2] in (72, 144) for c in seeds)
+    # 16 x 1 tiles of 64 x 64 on 256 compute units: K is split across workgroups in a third of the points
+    _, _, seeds = seeds_of("conv2d_yolo14_(1, 1024, 7, 7, 1024, 3, 1, 1, 1, 1)_rocm(0)")
+    splits = [c["reduce"][0][0] for c in seeds]
+    assert sum(1 for s in splits if s > 1) == 8 and max(splits) <= 16
+    assert any(c["reorder"][0][2] > 0 for c in seeds)            # K streaming is among them as well
+    # plenty of tiles: no K split
+    _, _, seeds = seeds_of(I8)
+    assert all(c["reduce"][0][0] == 1 for c in seeds)

@@ -73,6 +73,10 @@ int ftr_compile_to_code(const char *src, const char *arch,
                         size_t *size_out) {
     if (!src || !arch || !code_out || !size_out)
         return fail("ftr_compile_to_code: null argument");
+    if (nopts < 0 || (nopts > 0 && !opts))
+        return fail("ftr_compile_to_code: %d options but no option array", nopts);
+    for (int i = 0; i < nopts; ++i)
+        if (!opts[i]) return fail("ftr_compile_to_code: option %d is null", i);
     *code_out = nullptr;
     *size_out = 0;
     hiprtcProgram prog;

@@ -51,6 +51,10 @@ def test_null_arguments_fail_cleanly():
     L = rt.lib()
     assert L.ftr_compile_to_code(None, b"gfx950", None, 0, None, None) != 0
     assert b"null" in L.ftr_last_error()
+    code, size = ctypes.c_void_p(), ctypes.c_size_t()
+    src = b'extern "C" __global__ void k() {}'
+    assert L.ftr_compile_to_code(src, b"gfx950", None, 2, ctypes.byref(code), ctypes.byref(size)) != 0
+    assert b"option" in L.ftr_last_error() and not code.value
     ms = ctypes.c_float()
     assert L.ftr_time_seq(None, 1, 1, 0, 1, None, ctypes.byref(ms)) != 0
     assert L.ftr_module_attrs(None, None, None, None, None) != 0

@@ -288,7 +288,7 @@ class Scheduler(object):
             pass
         try:
             from .tuned import lookup
-            shipped = lookup(self.task_key) if self.warm_start else None
+            shipped = lookup(self.task_key, similar=True) if self.warm_start else None
             if shipped is not None and self.op_pos < len(shipped.op_config_lst):
                 candidates.append(shipped.op_config_lst[self.op_pos])
         except Exception:  # noqa: BLE001
@@ -719,7 +719,7 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
         if kwargs.get("warm_start", True):
             try:
                 from .tuned import lookup
-                shipped = lookup(task_key)
+                shipped = lookup(task_key, similar=True)
                 if shipped is not None and shipped.graph_config and \
                         len(shipped.graph_config.get("special") or []) == len(task.special_space):
                     configs = Config([], dict(shipped.graph_config))

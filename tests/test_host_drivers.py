@@ -112,3 +112,28 @@ def test_tuned_convolution_points_carry_over_to_the_im2col_form():
     d, _ = schedule_with_config(direct, lookup(direct))
     assert [k.defines for k in s.specs] == [k.defines for k in d.specs] and not s.intermediates
     assert lookup("gemm_conv2d_nothing_(1,)_rocm(0)") is None
+
+
+def test_layer_tuned_at_another_batch_size_seeds_the_search():
+    """lookup(similar=True): the same convolution layer at another batch lends
+    its tile, K division and pipeline; only the N grid level follows the batch.
+    Plain lookup() stays exact."""
+    from flextensor_amd.task import register, conv2d
+    args = (4, 256, 56, 56, 512, 3, 1, 1, 1, 1)
+    key = "conv2d_t_%s_rocm(0)" % str(args)
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    assert lookup(key) is None
+    lent = lookup(key, similar=True)
+    assert lent is not None and len(lent.op_config_lst) == 2
+    grid, waves, reps, mfma = lent.op_config_lst[1]["spatial"][1]
+    assert grid == -(-4 * 56 * 56 // (waves * reps * mfma))
+    sources = [lookup("conv2d_yolo5_(1, 256, 56, 56, 512, 3, 1, 1, 1, 1)_rocm(0)"),
+               lookup("conv2d_yolo_b85_(8, 256, 56, 56, 512, 3, 1, 1, 1, 1)_rocm(0)")]
+    assert any(lent.op_config_lst[1]["reduce"] == s.op_config_lst[1]["reduce"] and
+               lent.op_config_lst[1]["spatial"][0] == s.op_config_lst[1]["spatial"][0] for s in sources)
+    s, _ = schedule_with_config(key, lent)            # it lowers for the new batch
+    assert s.specs[-1].defines["N"] == 4 * 56 * 56
+    # nothing to lend: another layer, a depthwise task, a malformed key
+    assert lookup("conv2d_t_(4, 250, 56, 56, 512, 3, 1, 1, 1, 1)_rocm(0)", similar=True) is None
+    assert lookup("conv2d_depthwise_(4, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)", similar=True) is None
+    assert lookup("not a key", similar=True) is None

@@ -1,0 +1,57 @@
+"""The distance between the last MFMA of the main loop and the first read of
+its result registers, checked in the generated ISA (no GPU needed).
+
+A 16-pass MFMA's results may not be read for 19 issue slots and the hardware
+does not interlock. In the segment loop of balanced K streaming the compiler's
+padding missed the short branch from the main loop to the tile store; the
+templates therefore place the slots themselves. This test compiles the
+configuration that once failed and looks at the instruction stream."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from flextensor_amd.scheduler import schedule_with_config
+from flextensor_amd.task import TASK_TABLE  # noqa: F401  (registers the tasks)
+from flextensor_amd.utils import Config, ceil_div
+
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+KEYS = ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]
+
+
+def _isa(spec, tmp_path):
+    src = tmp_path / "kernel.hip"
+    src.write_text(spec.source())
+    out = tmp_path / "kernel.s"
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-S", "--cuda-device-only", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-include", "hip/hip_runtime.h", "-o", str(out), str(src)] + spec.options()
+    subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
+    return out.read_text().split("\n")
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_k_streaming_tile_store_waits_for_the_last_mfma(tmp_path):
+    key = "conv2d_baseline2_(8, 512, 7, 7, 2048, 1, 1, 0, 1, 1)_rocm(0)"
+    M, N, K = 2048, 392, 512
+    c = {k: [] for k in KEYS}
+    c["spatial"] = [[ceil_div(M, 64), 2, 1, 32], [ceil_div(N, 32), 1, 1, 32]]
+    c["reduce"], c["unroll"], c["fuse"], c["reorder"] = [[1, K // 64, 64]], [[5, 1]], [[1]], [[0, 0, 1]]
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[1, 0]], [[-1, 0]]
+    plan, _ = schedule_with_config(key, Config([{k: [] for k in KEYS}, c], g))
+    spec = plan.specs[-1]
+    assert spec.defines["SK_PER"] > 0 and spec.defines["DTL"] == 1 and spec.defines["MFMA"] == 32
+    lines = _isa(spec, tmp_path)
+    mfma = [i for i, l in enumerate(lines) if "v_mfma_f32_32x32x2" in l]
+    assert mfma, "no MFMA in the kernel"
+    last = mfma[-1]
+    nop = [i for i, l in enumerate(lines) if re.search(r"\bs_nop 15\b", l) and i > last]
+    reads = [i for i, l in enumerate(lines) if "v_accvgpr_read" in l and i > last]
+    assert nop and reads
+    # the explicit slots (16 + 4) stand between the loop and every later accumulator read
+    assert re.search(r"\bs_nop 3\b", lines[nop[0] + 1])
+    assert last < nop[0] < reads[0]
+    # and nothing reads an accumulator between the loop's first MFMA and its last
+    assert not [i for i, l in enumerate(lines) if "v_accvgpr_read" in l and mfma[0] < i < last]

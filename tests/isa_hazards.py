@@ -1,0 +1,114 @@
+"""Static check of generated gfx950 ISA for one software-managed hazard: a
+read of an MFMA's result registers before the matrix core has written them.
+
+The hardware does not interlock this case; the compiler pads it with s_nop,
+but its padding follows the control-flow graph with a visited set per block
+and can lose a short path. This module rebuilds the graph from the assembly
+text and walks every path forward from each MFMA for the required number of
+issue slots (test helper, not part of the package)."""
+import re
+
+# issue slots before another instruction may read the result: passes + 2 for the fp32
+# shapes, passes + 3 for the integer ones on gfx950 (taken with 16 and 8 passes, an upper bound)
+NEED = {"f32_32x32x2": 18, "f32_16x16x4": 10, "i32_32x32x32": 19, "i32_16x16x64": 11}
+REG = re.compile(r"\b([av])(?:\[(\d+):(\d+)\]|(\d+)\b)")
+BRANCH = re.compile(r"^s_(branch|cbranch_\w+)\s+(\S+)")
+
+
+def _regs(text):
+    out = set()
+    for m in REG.finditer(text):
+        kind = m.group(1)
+        if m.group(4) is not None:
+            out.add((kind, int(m.group(4))))
+        else:
+            out.update((kind, i) for i in range(int(m.group(2)), int(m.group(3)) + 1))
+    return out
+
+
+def parse(asm_text, kernel):
+    """Instructions of one kernel: list of (mnemonic, operand text), label -> index."""
+    lines = asm_text.split("\n")
+    start = next(i for i, l in enumerate(lines) if l.startswith(kernel + ":"))
+    insts, labels = [], {}
+    for l in lines[start + 1:]:
+        s = l.split(";")[0].strip()
+        if l.startswith(".Lfunc_end") or s.startswith(".Lfunc_end") or s == "s_endpgm" and False:
+            break
+        if not s:
+            continue
+        if s.endswith(":"):
+            labels[s[:-1]] = len(insts)
+            continue
+        if s.startswith("."):
+            continue
+        parts = s.split(None, 1)
+        insts.append((parts[0], parts[1] if len(parts) > 1 else ""))
+    return insts, labels
+
+
+def _slots(inst):
+    if inst[0] == "s_nop":
+        return int(inst[1].strip(), 0) + 1
+    return 1
+
+
+def _reads(inst):
+    """Registers an instruction reads (every operand but the destination of
+    an instruction that has one; stores and MFMA sources read all of theirs)."""
+    name, ops = inst
+    if not ops:
+        return set()
+    parts = [p.strip() for p in ops.split(",")]
+    if name.startswith(("global_store", "buffer_store", "ds_write", "flat_store", "scratch_store", "global_atomic")):
+        return _regs(ops)
+    return _regs(",".join(parts[1:]))
+
+
+def find_early_reads(asm_text, kernel):
+    """List of (mfma index, reader index, slots between) for reads that come too early."""
+    insts, labels = parse(asm_text, kernel)
+    found = []
+    for i, (name, ops) in enumerate(insts):
+        if not name.startswith("v_mfma"):
+            continue
+        shape = next((k for k in NEED if k in name), None)
+        if shape is None:
+            raise ValueError("unknown MFMA shape: " + name)
+        need = NEED[shape]
+        dst = _regs(ops.split(",")[0])
+        # walk forward over every path until `need` slots have passed
+        stack, seen = [(i + 1, 0)], {}
+        while stack:
+            j, used = stack.pop()
+            while j < len(insts) and used < need:
+                if seen.get(j, need + 1) <= used:
+                    break
+                seen[j] = used
+                jn, jo = insts[j]
+                if jn.startswith("v_mfma"):
+                    # the next MFMA: reading the result as its own accumulator is interlocked;
+                    # as a multiplicand it is not
+                    parts = [p.strip() for p in jo.split(",")]
+                    if _regs(",".join(parts[1:3])) & dst:
+                        found.append((i, j, used))
+                    if _regs(parts[0]) & dst:
+                        break        # the registers get a new producer: this walk ends
+                elif _reads((jn, jo)) & dst:
+                    found.append((i, j, used))
+                    break
+                elif jn.startswith(("v_", "ds_read", "global_load", "buffer_load")) and _regs(jo.split(",")[0]) & dst \
+                        and _regs(jo.split(",")[0]) >= dst:
+                    break            # overwritten entirely
+                b = BRANCH.match(jn + " " + jo)
+                used += _slots((jn, jo))
+                if b:
+                    target = labels.get(b.group(2))
+                    if target is not None:
+                        stack.append((target, used))
+                    if b.group(1) == "branch":
+                        break
+                if jn == "s_endpgm":
+                    break
+                j += 1
+    return found, insts

@@ -13,6 +13,8 @@ import subprocess
 
 import pytest
 
+import isa_hazards
+
 from flextensor_amd.scheduler import schedule_with_config
 from flextensor_amd.task import TASK_TABLE  # noqa: F401  (registers the tasks)
 from flextensor_amd.utils import Config, ceil_div
@@ -55,3 +57,53 @@ def test_k_streaming_tile_store_waits_for_the_last_mfma(tmp_path):
     assert last < nop[0] < reads[0]
     # and nothing reads an accumulator between the loop's first MFMA and its last
     assert not [i for i, l in enumerate(lines) if "v_accvgpr_read" in l and mfma[0] < i < last]
+    # every path from every MFMA, with the control-flow graph rebuilt from the text
+    found, _ = isa_hazards.find_early_reads("\n".join(lines), "igemm_f32")
+    assert found == []
+
+
+SNIPPET = """
+k:
+	v_mfma_f32_32x32x2_f32 a[0:15], v1, v2, a[0:15]
+	s_cbranch_scc1 .LBB0_2
+	s_nop 15
+	s_nop 1
+	v_accvgpr_read_b32 v3, a15
+	s_endpgm
+.LBB0_2:
+	s_add_i32 s0, s0, 1
+%s	v_accvgpr_read_b32 v4, a0
+	s_endpgm
+.Lfunc_end0:
+"""
+
+
+def test_checker_follows_branches_and_counts_nops():
+    found, insts = isa_hazards.find_early_reads(SNIPPET % "", "k")
+    assert [(insts[j][1], used) for _, j, used in found] == [("v4, a0", 2)]       # the padded fall-through passes
+    found, _ = isa_hazards.find_early_reads(SNIPPET % "\ts_nop 15\n", "k")
+    assert found == []
+    # the next MFMA may accumulate onto the result at once, but not multiply with it
+    chain = "k:\n\tv_mfma_f32_16x16x4_f32 v[0:3], v8, v9, v[0:3]\n\tv_mfma_f32_16x16x4_f32 v[0:3], v8, v9, v[0:3]\n" \
+            "\tv_mfma_f32_16x16x4_f32 v[4:7], v0, v9, v[4:7]\n\ts_endpgm\n.Lfunc_end0:\n"
+    found, insts = isa_hazards.find_early_reads(chain, "k")
+    assert [(i, j) for i, j, _ in found] == [(1, 2)]
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_benchmark_kernels_have_no_early_accumulator_reads(tmp_path):
+    """Every MFMA kernel of the shipped benchmark configurations, all paths."""
+    import __graft_entry__ as g
+    from flextensor_amd.tuned import lookup
+    checked = 0
+    for n, key in enumerate(g.BENCH_KEYS):
+        plan, _ = schedule_with_config(key, lookup(key))
+        for spec in plan.specs:
+            if spec.kernel not in ("igemm_f32", "gemm_i8"):
+                continue
+            d = tmp_path / str(n)
+            d.mkdir()
+            found, insts = isa_hazards.find_early_reads("\n".join(_isa(spec, d)), spec.kernel)
+            assert found == [], (key, [(insts[i], insts[j], used) for i, j, used in found[:3]])
+            checked += 1
+    assert checked == 5

@@ -5,8 +5,17 @@ The hardware does not interlock this case; the compiler pads it with s_nop,
 but its padding follows the control-flow graph with a visited set per block
 and can lose a short path. This module rebuilds the graph from the assembly
 text and walks every path forward from each MFMA for the required number of
-issue slots (test helper, not part of the package)."""
+issue slots.
+
+    python -m flextensor_amd.isa_check [tuned.log]     # every MFMA kernel of a key:json log
+
+needs hipcc (the kernels are compiled to assembly text on the host; no GPU)."""
+import os
 import re
+import shutil
+import subprocess
+import sys
+import tempfile
 
 # issue slots before another instruction may read the result: passes + 2 for the fp32
 # shapes, passes + 3 for the integer ones on gfx950 (taken with 16 and 8 passes, an upper bound)
@@ -112,3 +121,59 @@ def find_early_reads(asm_text, kernel):
                     break
                 j += 1
     return found, insts
+
+
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+def assembly_of(spec, workdir=None):
+    """Assembly text of one KernelSpec for gfx950 (hipcc -S with the options hiprtc gets)."""
+    d = workdir or tempfile.mkdtemp(prefix="ft_isa_")
+    src, out = os.path.join(d, "kernel.hip"), os.path.join(d, "kernel.s")
+    with open(src, "w") as f:
+        f.write(spec.source())
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-S", "--cuda-device-only", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-include", "hip/hip_runtime.h", "-o", out, src] + spec.options()
+    subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
+    with open(out) as f:
+        text = f.read()
+    if workdir is None:
+        shutil.rmtree(d, ignore_errors=True)
+    return text
+
+
+def check_plan(plan):
+    """[(kernel, mfma instruction, reading instruction, slots between)] over the MFMA kernels of a plan."""
+    out = []
+    for spec in plan.specs:
+        if spec.kernel not in ("igemm_f32", "gemm_i8"):
+            continue
+        found, insts = find_early_reads(assembly_of(spec), spec.kernel)
+        out.extend((spec.kernel, insts[i], insts[j], used) for i, j, used in found)
+    return out
+
+
+def main(argv):
+    from .scheduler import schedule_with_config
+    from .task import TASK_TABLE
+    from .tuned import LOG, load
+    table = load(argv[1] if len(argv) > 1 else LOG)
+    seen, bad = set(), 0
+    for key, cfg in table.items():
+        if key not in TASK_TABLE:
+            print("skipped (not registered):", key)
+            continue
+        plan, _ = schedule_with_config(key, cfg)
+        sig = tuple((sp.template, tuple(sp.options())) for sp in plan.specs)
+        if sig in seen:
+            continue
+        seen.add(sig)
+        for kernel, mfma, reader, used in check_plan(plan):
+            bad += 1
+            print("EARLY READ %s %s: %s %s -> %s %s after %d slots" % ((key, kernel) + mfma + reader + (used,)))
+    print("%d plans checked, %d early reads" % (len(seen), bad))
+    return 1 if bad else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv))

@@ -13,7 +13,7 @@ import subprocess
 
 import pytest
 
-import isa_hazards
+from flextensor_amd import isa_check as isa_hazards
 
 from flextensor_amd.scheduler import schedule_with_config
 from flextensor_amd.task import TASK_TABLE  # noqa: F401  (registers the tasks)

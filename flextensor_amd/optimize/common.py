@@ -4,7 +4,8 @@ Same roles and command-line flags as the reference's
 flextensor/optimize/common.py (evaluate :17-60, test :63-82,
 init_arg_parser :85-114). ``--check`` compares the tuned kernels with the
 plain default-schedule kernels of the same task on the device, which is what
-the reference's ``check_result`` does with the default llvm build.
+the reference's ``check_result`` does with the default llvm build, and runs
+the static check of the kernels' assembly (isa_check).
 """
 import sys
 
@@ -38,6 +39,12 @@ def test(task_key, configs, dev_id=None, rpc_info=None, check_result=False):
         ok, metric = m.check(m.sets[0][-1])
         built.close()
         print("Test correctness...", "passed!" if ok else "failed!", "metric", metric)
+        # and the assembly: no read of an MFMA's result before the matrix core has written it
+        from .. import isa_check
+        import os
+        if os.path.exists(isa_check.HIPCC):
+            early = isa_check.check_plan(s)
+            print("Test instruction stream...", "passed!" if not early else "failed! %s" % (early[:2],))
     print(task_key, "use", time_cost, "ms")
     print()
     return time_cost

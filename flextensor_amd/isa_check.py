@@ -1,5 +1,6 @@
 """Static check of generated gfx950 ISA for one software-managed hazard: a
-read of an MFMA's result registers before the matrix core has written them.
+read (or an overwrite by another instruction) of an MFMA's result registers
+before the matrix core has written them.
 
 The hardware does not interlock this case; the compiler pads it with s_nop,
 but its padding follows the control-flow graph with a visited set per block
@@ -106,9 +107,12 @@ def find_early_reads(asm_text, kernel):
                 elif _reads((jn, jo)) & dst:
                     found.append((i, j, used))
                     break
-                elif jn.startswith(("v_", "ds_read", "global_load", "buffer_load")) and _regs(jo.split(",")[0]) & dst \
-                        and _regs(jo.split(",")[0]) >= dst:
-                    break            # overwritten entirely
+                elif jn.startswith(("v_", "ds_read", "global_load", "buffer_load")) and not jn.startswith("v_cmp") \
+                        and _regs(jo.split(",")[0]) & dst:
+                    # another instruction writes a result register while the MFMA may still be
+                    # writing it: the same distance applies to this write-after-write
+                    found.append((i, j, used))
+                    break
                 b = BRANCH.match(jn + " " + jo)
                 used += _slots((jn, jo))
                 if b:

@@ -88,6 +88,12 @@ def test_checker_follows_branches_and_counts_nops():
             "\tv_mfma_f32_16x16x4_f32 v[4:7], v0, v9, v[4:7]\n\ts_endpgm\n.Lfunc_end0:\n"
     found, insts = isa_hazards.find_early_reads(chain, "k")
     assert [(i, j) for i, j, _ in found] == [(1, 2)]
+    # an early overwrite of the result registers by another instruction counts as well
+    waw = "k:\n\tv_mfma_f32_16x16x4_f32 a[0:3], v8, v9, a[0:3]\n\ts_nop 3\n\tv_accvgpr_write_b32 a2, 0\n\ts_endpgm\n.Lfunc_end0:\n"
+    found, _ = isa_hazards.find_early_reads(waw, "k")
+    assert [(i, j, used) for i, j, used in found] == [(0, 2, 4)]
+    found, _ = isa_hazards.find_early_reads(waw.replace("s_nop 3", "s_nop 9"), "k")
+    assert found == []
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")

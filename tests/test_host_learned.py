@@ -151,3 +151,26 @@ def test_schedule_use_model_measures_the_models_choice(tmp_path):
     # the device (here: the cost function) is only asked for seeds and for the model's final candidates
     assert 0 < len(measured) <= 2 * (24 + 10)      # per level: heuristic seeds + the model's final ten
     assert math.isfinite(_cost(GEMM, configs, None, 1))
+
+
+def test_schedule_method_q_on_the_four_operator_im2col_graph(tmp_path):
+    """method="q" over [Padding, Img2Col, ComputeGemm, Col2Img]: only the GEMM
+    has knobs, the graph level decides which stages exist as kernels (host
+    cost: one unit per kernel plus the GEMM's synthetic cost)."""
+    from flextensor_amd.scheduler import schedule_with_config
+    np.random.seed(7)
+    torch.manual_seed(7)
+    key = "gemm_conv2d_yolo7_(1, 256, 28, 28, 512, 3, 1, 1, 1, 1)_rocm(0)"
+
+    def cost(task_key, cfg, op_pos, number):
+        plan = schedule_with_config(task_key, cfg, op_pos=op_pos)[0]
+        d = [sp for sp in plan.specs if sp.kernel == "igemm_f32"][0].defines
+        tile = d["WAVES_M"] * d["REP_M"] * d["WAVES_N"] * d["REP_N"] * d["MFMA"] ** 2
+        return len(plan.specs) + abs(np.log2(tile / 8192.0)) + (0.0 if d["BK"] in (72, 144) else 0.5)
+
+    s, bufs, configs = schedule(key, op_trial=6, op_stop=6, graph_trial=3, parallel=4, method="q", evaluator=cost,
+                                warm_up=(1, 6), verbose=False, perf_path=str(tmp_path), trials=[1, 1, 6, 1],
+                                warm_start=False)
+    assert len(configs.op_config_lst) == 4 and configs.op_config_lst[2]["spatial"]
+    assert [sp.kernel for sp in s.specs] == ["igemm_f32"]            # folded: fewest kernels wins
+    assert configs.graph_config["inline"][0][:2] == [1, 1] and configs.graph_config["merge"][0][3] == 1

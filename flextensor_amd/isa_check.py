@@ -1,6 +1,12 @@
-"""Static check of generated gfx950 ISA for one software-managed hazard: a
-read (or an overwrite by another instruction) of an MFMA's result registers
-before the matrix core has written them.
+"""Static checks of generated gfx950 ISA.
+
+1. A software-managed hazard: a read (or an overwrite by another instruction)
+of an MFMA's result registers before the matrix core has written them.
+2. The hand-off of balanced K streaming: on every path from a store to a
+workspace slot (a device-scope store, ``sc1``) to the next arrival count (a
+``global_atomic_add``) the wavefront waits for its stores (``s_waitcnt``
+with ``vmcnt(0)``) and then passes an ``s_barrier``; neither a barrier nor a
+workgroup-scope fence waits for vector stores by itself.
 
 The hardware does not interlock this case; the compiler pads it with s_nop,
 but its padding follows the control-flow graph with a visited set per block
@@ -127,6 +133,54 @@ def find_early_reads(asm_text, kernel):
     return found, insts
 
 
+def _successors(insts, labels, j):
+    """Indices control can reach from instruction j."""
+    name, ops = insts[j]
+    if name == "s_endpgm":
+        return []
+    b = BRANCH.match(name + " " + ops)
+    out = []
+    if b:
+        target = labels.get(b.group(2))
+        if target is not None:
+            out.append(target)
+        if b.group(1) == "branch":
+            return out
+    if j + 1 < len(insts):
+        out.append(j + 1)
+    return out
+
+
+def find_unordered_arrivals(asm_text, kernel):
+    """[(slot store index, arrival index)] for arrival counts that a slot store can
+    reach without the wavefront having waited for its stores and passed a barrier."""
+    insts, labels = parse(asm_text, kernel)
+    found = []
+    for i, (name, ops) in enumerate(insts):
+        if not (name.startswith("global_store") and re.search(r"\bsc1\b", ops)):
+            continue
+        # stage 0: store outstanding; 1: waited for; 2: waited for and a barrier passed
+        stack, seen = [(j, 0) for j in _successors(insts, labels, i)], set()
+        while stack:
+            j, stage = stack.pop()
+            if (j, stage) in seen:
+                continue
+            seen.add((j, stage))
+            jn, jo = insts[j]
+            if jn.startswith("global_atomic_add"):
+                if stage < 2:
+                    found.append((i, j))
+                continue                      # the arrival is counted: this walk ends
+            if jn.startswith("global_store") and re.search(r"\bsc1\b", jo):
+                stage = 0                     # a later slot store is outstanding again
+            elif jn == "s_waitcnt" and re.search(r"\bvmcnt\(0\)", jo):
+                stage = max(stage, 1)
+            elif jn == "s_barrier" and stage == 1:
+                stage = 2
+            stack.extend((k, stage) for k in _successors(insts, labels, j))
+    return found, insts
+
+
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
@@ -147,13 +201,19 @@ def assembly_of(spec, workdir=None):
 
 
 def check_plan(plan):
-    """[(kernel, mfma instruction, reading instruction, slots between)] over the MFMA kernels of a plan."""
+    """[(kernel, first instruction, second instruction, detail)] over the MFMA kernels of a plan:
+    early reads of MFMA results (detail = issue slots between) and arrival counts of the
+    K-streaming exchange that do not wait for the slot stores (detail = "arrival")."""
     out = []
     for spec in plan.specs:
         if spec.kernel not in ("igemm_f32", "gemm_i8"):
             continue
-        found, insts = find_early_reads(assembly_of(spec), spec.kernel)
+        text = assembly_of(spec)
+        found, insts = find_early_reads(text, spec.kernel)
         out.extend((spec.kernel, insts[i], insts[j], used) for i, j, used in found)
+        if spec.defines.get("SK_PER", 0):
+            found, insts = find_unordered_arrivals(text, spec.kernel)
+            out.extend((spec.kernel, insts[i], insts[j], "arrival") for i, j in found)
     return out
 
 
@@ -174,8 +234,11 @@ def main(argv):
         seen.add(sig)
         for kernel, mfma, reader, used in check_plan(plan):
             bad += 1
-            print("EARLY READ %s %s: %s %s -> %s %s after %d slots" % ((key, kernel) + mfma + reader + (used,)))
-    print("%d plans checked, %d early reads" % (len(seen), bad))
+            if used == "arrival":
+                print("UNORDERED ARRIVAL %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
+            else:
+                print("EARLY READ %s %s: %s %s -> %s %s after %d slots" % ((key, kernel) + mfma + reader + (used,)))
+    print("%d plans checked, %d findings" % (len(seen), bad))
     return 1 if bad else 0
 
 

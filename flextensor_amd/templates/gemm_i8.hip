@@ -290,7 +290,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         auto dma16 = [&](const i32x4& rsrc, const signed char* dst, unsigned vo, int so) {
             const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory");
+                         :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
         };
         auto dma_tile = [&](int kt, int buf) {
             const int k0 = kt * BK;

@@ -557,6 +557,10 @@ CONV_CASES = [
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, ks=1)),        # groups 4, K streaming
     ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16, ks=1, st=3)),   # K streaming, padded K
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32, ks=2)),          # 1x1, K streaming
+    # 98 tiles of 36 k-steps over 256 workgroups: most tiles have three sharers and most workgroups
+    # end one tile and begin the next (an early version of the exchange summed this one wrong)
+    ((1, 64, 56, 56, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=2, wn=2, rn=1, mf=16, bk=16, st=3, ks=1)),
+    ((1, 64, 56, 56, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=2, wn=2, rn=1, mf=16, bk=16, st=2, ks=2)),
 ]
 
 

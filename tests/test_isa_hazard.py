@@ -113,3 +113,55 @@ def test_benchmark_kernels_have_no_early_accumulator_reads(tmp_path):
             assert found == [], (key, [(insts[i], insts[j], used) for i, j, used in found[:3]])
             checked += 1
     assert checked == 5
+
+
+ARRIVAL = """
+k:
+	global_store_dword v1, v2, s[0:1] sc1
+	s_cbranch_scc1 .LBB0_2
+%s	s_barrier
+	global_atomic_add v3, v4, v5, s[2:3] sc0
+	s_endpgm
+.LBB0_2:
+	s_waitcnt vmcnt(0)
+	s_barrier
+	global_atomic_add v3, v4, v5, s[2:3] sc0
+	s_endpgm
+.Lfunc_end0:
+"""
+
+
+def test_arrival_checker_wants_a_wait_then_a_barrier_on_every_path():
+    found, insts = isa_hazards.find_unordered_arrivals(ARRIVAL % "", "k")
+    assert [(i, insts[j][0]) for i, j in found] == [(0, "global_atomic_add")] and found[0][1] == 3
+    found, _ = isa_hazards.find_unordered_arrivals(ARRIVAL % "\ts_waitcnt lgkmcnt(0)\n", "k")
+    assert len(found) == 1                                    # a wait for LDS only does not count
+    found, _ = isa_hazards.find_unordered_arrivals(ARRIVAL % "\ts_waitcnt vmcnt(0) lgkmcnt(0)\n", "k")
+    assert found == []
+    # the wait has to come before the barrier, not after it
+    late = ARRIVAL.replace("%s\ts_barrier\n", "\ts_barrier\n\ts_waitcnt vmcnt(0)\n")
+    found, _ = isa_hazards.find_unordered_arrivals(late, "k")
+    assert len(found) == 1
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_k_streaming_arrivals_wait_for_the_slot_stores(tmp_path):
+    """Both ways a tile can travel to LDS, on the shipped K-streaming entry and on a
+    register-staged variant of it: every slot store is waited for before its arrival is
+    counted, in the run's last segment and in the prologue of a following one."""
+    from flextensor_amd.tuned import lookup
+    key = "conv2d_baseline1_(8, 256, 14, 14, 512, 3, 1, 1, 1, 1)_rocm(0)"
+    shipped = lookup(key)
+    staged = Config([dict(c) for c in shipped.op_config_lst], dict(shipped.graph_config))
+    staged.op_config_lst[1]["unroll"] = [[3, 1]]
+    staged.op_config_lst[1]["reduce"] = [[1, 72, 32]]
+    for n, cfg in enumerate((shipped, staged)):
+        plan, _ = schedule_with_config(key, cfg)
+        spec = plan.specs[-1]
+        assert spec.defines["SK_PER"] > 0
+        d = tmp_path / str(n)
+        d.mkdir()
+        text = "\n".join(_isa(spec, d))
+        assert re.search(r"global_store_dword.*sc1", text) and "global_atomic_add" in text
+        found, insts = isa_hazards.find_unordered_arrivals(text, spec.kernel)
+        assert found == [], [(insts[i], insts[j]) for i, j in found[:3]]

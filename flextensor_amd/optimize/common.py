@@ -132,7 +132,8 @@ def run_driver(args, shapes, make_task, describe):
                 if value:
                     print(name, value)
             time_cost = evaluate(task.key, s, bufs, args.target, args.device, 100, rpc_info)
-            print("# %.5f ms" % time_cost, file=flog, flush=True)
+            # the log holds nothing but key:json lines, so the reference's readers
+            # (line.split(":", 1) + json.loads on every line) take it as it is
             print(task.key + ":" + json.dumps(configs), file=flog, flush=True)
             print("Use", time_cost, "ms")
             print("Cost", endt - beg, "s")

@@ -414,7 +414,17 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     if dtl and stages > 2 and ((bm * bk // av) % nt or ((bn * bk) // bv) % nt or (stages - 2) * (ea + eb) > 63):
         raise InvalidConfig("more than two direct-to-LDS buffers need whole rounds of loads per tile, "
                             "at most 63 of them in flight")
-    if max(view.M * view.K, view.K * view.N, view.M * view.N) * view.groups * 4 >= 2 ** 31:
+    # bytes behind the two buffer descriptors (A_BYTES / B_BYTES of the template) and of C: in MODE 1
+    # B is the image itself, larger than K x N when the stride exceeds the kernel, and larger
+    # still once the padding is materialised
+    a_bytes = view.groups * view.M * view.K * 4
+    if view.mode == 1:
+        cv = view.conv
+        grow = 2 * cv["CPAD"] if materialized_pad else 0
+        b_bytes = cv["CB"] * cv["CC"] * (cv["CH"] + grow) * (cv["CW"] + grow) * 4
+    else:
+        b_bytes = view.groups * view.K * view.N * 4
+    if max(a_bytes, b_bytes, view.groups * view.M * view.N * 4) >= 2 ** 31:
         raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
     D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
     if dtl:

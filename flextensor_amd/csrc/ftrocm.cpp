@@ -7,6 +7,7 @@
 // time_evaluator). Nothing here computes on the CPU.
 
 #include "ftrocm.h"
+#include "ftrocm_internal.h"
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
@@ -27,15 +28,7 @@ namespace {
 
 thread_local std::string g_err;
 
-int fail(const char *fmt, ...) {
-    char buf[4096];
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(buf, sizeof buf, fmt, ap);
-    va_end(ap);
-    g_err = buf;
-    return 1;
-}
+#define fail ftr_internal_fail
 
 #define FTR_HIP(call)                                                         \
     do {                                                                      \
@@ -49,6 +42,7 @@ int fail(const char *fmt, ...) {
 
 int launch_one(const ftr_launch_desc_t &d, hipStream_t s) {
     if (!d.mod) return fail("ftr_launch: null module");
+    if (!d.args) return fail("ftr_launch: null argument array");
     for (int i = 0; i < 3; ++i)
         if (d.grid[i] == 0 || d.block[i] == 0)
             return fail("ftr_launch: zero grid/block extent in dim %d", i);
@@ -61,6 +55,16 @@ int launch_one(const ftr_launch_desc_t &d, hipStream_t s) {
 }
 
 }  // namespace
+
+int ftr_internal_fail(const char *fmt, ...) {
+    char buf[4096];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return 1;
+}
 
 extern "C" {
 
@@ -142,6 +146,12 @@ int ftr_module_load(const void *code, size_t size, const char *kernel_name,
         (void)hipGetLastError();
         return fail("kernel '%s' not found in code object: %s", kernel_name,
                     hipGetErrorString(e));
+    }
+    // set-up time is also when the static workspace of this device is looked
+    // up, so that ftr_launch_seq_static_ws has nothing left to resolve later
+    if (ftr_internal_static_ws(nullptr)) {
+        (void)hipModuleUnload(m);
+        return 1;
     }
     ftr_module *mod = new ftr_module{m, f};
     *out = mod;

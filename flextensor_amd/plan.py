@@ -34,8 +34,8 @@ class KernelPlan(object):
         """Compile every kernel to a code object (no device needed)."""
         return [rt.compile_to_code(s.source(), s.options(), arch) for s in self.specs]
 
-    def build(self):
-        return BuiltPlan(self)
+    def build(self, static_workspace=False):
+        return BuiltPlan(self, static_workspace=static_workspace)
 
     def __repr__(self):
         return "KernelPlan(%s: %s)" % (self.task_key, ", ".join(s.kernel for s in self.specs))
@@ -61,7 +61,10 @@ def current_stream():
 class BuiltPlan(object):
     """Loaded kernels of a plan; call it with device tensors in ``bufs`` order."""
 
-    def __init__(self, plan):
+    def __init__(self, plan, static_workspace=False):
+        """``static_workspace=True`` keeps the plan's workspaces (K-streaming
+        slots and counters) in the runtime library's fixed device array instead
+        of allocating them, and calls go through ftr_launch_seq_static_ws."""
         import torch
         if not torch.cuda.is_available():
             raise rt.RuntimeError_("no GPU visible: a kernel plan can only be built on a device")
@@ -72,8 +75,24 @@ class BuiltPlan(object):
         self.scratch = {}
         for name, (shape, dtype) in plan.intermediates.items():
             self.scratch[name] = torch.empty(shape, dtype=_torch_dtype(dtype), device="cuda")
-        for name, (shape, dtype) in plan.workspaces.items():
-            self.scratch[name] = torch.zeros(shape, dtype=_torch_dtype(dtype), device="cuda")
+        self.static_layout = None
+        if static_workspace:
+            # name -> (offset, bytes, zero): consecutive 256-byte aligned ranges; the
+            # arrival counters must start at zero, the slots are written before they are read
+            self.static_layout, offset = {}, 0
+            for name, (shape, dtype) in sorted(plan.workspaces.items()):
+                n = 1
+                for d in shape:
+                    n *= int(d)
+                nbytes = (n * {"float32": 4, "int32": 4, "int8": 1}[dtype] + 15) // 16 * 16
+                self.static_layout[name] = (offset, nbytes, 0 if name.endswith("_parts") else 1)
+                offset = (offset + nbytes + 255) // 256 * 256
+            if offset > rt.STATIC_WS_BYTES:
+                raise rt.RuntimeError_("the plan's workspaces need %d bytes, the static workspace holds %d"
+                                       % (offset, rt.STATIC_WS_BYTES))
+        else:
+            for name, (shape, dtype) in plan.workspaces.items():
+                self.scratch[name] = torch.zeros(shape, dtype=_torch_dtype(dtype), device="cuda")
 
     def attrs(self):
         return [m.attrs() for m in self.modules]
@@ -97,10 +116,14 @@ class BuiltPlan(object):
         named = dict(zip(self.plan.buf_names, tensors))
         named.update(self.scratch)
         out = []
-        for spec, mod in zip(self.plan.specs, self.modules):
+        self._binds = []
+        for li, (spec, mod) in enumerate(zip(self.plan.specs, self.modules)):
             vals = []
-            for kind, v in spec.args:
-                if kind == "buf":
+            for ai, (kind, v) in enumerate(spec.args):
+                if kind == "buf" and self.static_layout is not None and v in self.static_layout:
+                    vals.append(ctypes.c_void_p(0))      # the library writes the address here
+                    self._binds.append((li, ai) + self.static_layout[v])
+                elif kind == "buf":
                     vals.append(rt.ptr(named[v]))
                 elif kind == "i32":
                     vals.append(ctypes.c_int(int(v)))
@@ -114,7 +137,11 @@ class BuiltPlan(object):
         return out
 
     def __call__(self, *tensors):
-        rt.launch_seq(self.launches(tensors), stream=current_stream())
+        launches = self.launches(tensors)
+        if self.static_layout is not None:
+            rt.launch_seq_static_ws(launches, self._binds, stream=current_stream())
+        else:
+            rt.launch_seq(launches, stream=current_stream())
 
     def time(self, tensor_sets, warmup=2, iters=10, warm_ms=0.0):
         """Mean ms per run, rotating through ``tensor_sets``.
@@ -123,6 +150,8 @@ class BuiltPlan(object):
         long first: after an idle period the clocks take on the order of
         100 ms of continuous work to reach their steady state, and a kernel
         timed before that reads 15-25 % slow."""
+        if self.static_layout is not None:
+            raise rt.RuntimeError_("timing runs over caller-owned workspaces: build without static_workspace")
         sets = [self.launches(ts) for ts in tensor_sets]
         stream = current_stream()
         if warm_ms > 0:

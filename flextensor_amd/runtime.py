@@ -26,7 +26,7 @@ ABI_VERSION = 1
 EXPORTS = (
     "ftr_abi_version", "ftr_last_error", "ftr_compile_to_code", "ftr_code_free",
     "ftr_module_load", "ftr_compile", "ftr_module_free", "ftr_module_attrs",
-    "ftr_launch", "ftr_launch_seq", "ftr_time", "ftr_time_seq",
+    "ftr_launch", "ftr_launch_seq", "ftr_launch_seq_static_ws", "ftr_time", "ftr_time_seq",
     "ftr_device_props", "ftr_device_count",
 )
 
@@ -61,6 +61,18 @@ class _LaunchDesc(ctypes.Structure):
         ("args", ctypes.POINTER(ctypes.c_void_p)),
     ]
 
+
+class _WsBind(ctypes.Structure):
+    _fields_ = [
+        ("launch", ctypes.c_int),
+        ("arg", ctypes.c_int),
+        ("offset", ctypes.c_size_t),
+        ("bytes", ctypes.c_size_t),
+        ("zero", ctypes.c_int),
+    ]
+
+
+STATIC_WS_BYTES = 64 << 20      # FTR_STATIC_WS_BYTES of include/ftrocm.h
 
 _lib = None
 _lib_lock = threading.Lock()
@@ -100,6 +112,8 @@ def lib():
             ctypes.c_void_p, ctypes.c_uint * 3, ctypes.c_uint * 3, ctypes.c_uint,
             ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p]
         L.ftr_launch_seq.argtypes = [ctypes.POINTER(_LaunchDesc), ctypes.c_int, ctypes.c_void_p]
+        L.ftr_launch_seq_static_ws.argtypes = [ctypes.POINTER(_LaunchDesc), ctypes.c_int,
+                                               ctypes.POINTER(_WsBind), ctypes.c_int, ctypes.c_void_p]
         L.ftr_time.argtypes = [
             ctypes.c_void_p, ctypes.c_uint * 3, ctypes.c_uint * 3, ctypes.c_uint,
             ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int,
@@ -160,6 +174,7 @@ def code_key(src, opts, arch=DEFAULT_ARCH):
 
 _worker = None
 _worker_lock = threading.Lock()
+WORKER_REPLY_MARK = "FTR-REPLY "
 
 
 def _stop_worker():
@@ -188,12 +203,18 @@ def _compile_out_of_process(src, opts, arch):
         _worker.stdin.write(json.dumps({"src": src, "opts": list(opts), "arch": arch,
                                         "cache_dir": CACHE_DIR}) + "\n")
         _worker.stdin.flush()
-        line = _worker.stdout.readline()
-    if not line:
-        raise RuntimeError_("compile server died")
-    rep = json.loads(line)
+        while True:
+            line = _worker.stdout.readline()
+            if not line:
+                raise RuntimeError_("compile server died")
+            if line.startswith(WORKER_REPLY_MARK):      # anything else is a library's chatter
+                break
+    rep = json.loads(line[len(WORKER_REPLY_MARK):])
     if not rep.get("ok"):
         raise RuntimeError_("ftr_compile_to_code: %s" % rep.get("error"))
+    if "b64" in rep:
+        import base64
+        return base64.b64decode(rep["b64"])
     with open(rep["path"], "rb") as f:
         return f.read()
 
@@ -353,6 +374,18 @@ def _desc_array(launches):
 def launch_seq(launches, stream=0):
     arr = _desc_array(launches)
     _check(lib().ftr_launch_seq(arr, len(launches), ctypes.c_void_p(stream)), "ftr_launch_seq")
+
+
+def launch_seq_static_ws(launches, binds, stream=0):
+    """``launch_seq`` with the workspace arguments bound to the library's
+    static device array instead of caller-owned buffers; allocates nothing.
+    ``binds`` = [(launch index, argument index, offset, bytes, zero)]."""
+    arr = _desc_array(launches)
+    b = (_WsBind * max(len(binds), 1))()
+    for dst, (launch, arg, offset, nbytes, zero) in zip(b, binds):
+        dst.launch, dst.arg, dst.offset, dst.bytes, dst.zero = int(launch), int(arg), int(offset), int(nbytes), int(zero)
+    _check(lib().ftr_launch_seq_static_ws(arr, len(launches), b, len(binds), ctypes.c_void_p(stream)),
+           "ftr_launch_seq_static_ws")
 
 
 def time_seq(sets, warmup=3, iters=20, stream=0):

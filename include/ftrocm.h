@@ -122,6 +122,38 @@ int ftr_time(ftr_module_t mod, const unsigned grid[3], const unsigned block[3],
 int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
                  int warmup, int iters, void *stream, float *ms_mean);
 
+/* Bytes of the static device workspace ftr_launch_seq_static_ws binds. */
+#define FTR_STATIC_WS_BYTES (64u << 20)
+
+/* One workspace argument of a launch sequence: the pointer-sized slot that
+ * seq[launch].args[arg] points at receives the device address of bytes
+ * [offset, offset + bytes) of the static workspace. offset must be a multiple
+ * of 256 and bytes a multiple of 16; with zero != 0 the range is cleared on
+ * the stream (by a fill kernel) before the first launch. */
+typedef struct ftr_ws_bind {
+    int launch;
+    int arg;
+    size_t offset;
+    size_t bytes;
+    int zero;
+} ftr_ws_bind_t;
+
+/* ftr_launch_seq for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference, whose runtime allocates freely. The
+ * workspace arguments named by `binds` (the per-tile slots and arrival
+ * counters of a K-streaming plan, which ftr_launch_seq takes as caller-owned
+ * buffers) are bound to a fixed FTR_STATIC_WS_BYTES array inside the
+ * library's device image; the caller still passes every input and output.
+ * Calls hipMalloc/hipFree never; fails with a message when a range does not
+ * fit. The array is one per GPU and keeps the previous call's contents: ask
+ * for zero where a kernel relies on zeros. Calls that overlap in time on one
+ * GPU (two streams, two threads) race on it. The array's address is resolved
+ * per device at ftr_module_load time. */
+int ftr_launch_seq_static_ws(const ftr_launch_desc_t *seq, int n,
+                             const ftr_ws_bind_t *binds, int nbinds,
+                             void *stream);
+
 /* Properties of device `dev`. Stands in for the tvm device queries in
  * flextensor/measure.py:10-20. */
 int ftr_device_props(int dev, ftr_props_t *out);

@@ -12,11 +12,13 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <thread>
 #include <vector>
 
 struct ftr_module {
@@ -230,16 +232,30 @@ int ftr_launch_seq(const ftr_launch_desc_t *seq, int n, void *stream) {
     return 0;
 }
 
-int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
-                 int warmup, int iters, void *stream, float *ms_mean) {
+int ftr_time_seq_deadline(const ftr_launch_desc_t *seqs, int n_per_iter,
+                          int nsets, int warmup, int iters, void *stream,
+                          double timeout_s, float *ms_mean) {
     if (!seqs || !ms_mean || n_per_iter < 1 || nsets < 1 || iters < 1 ||
-        warmup < 0)
+        warmup < 0 || !(timeout_s >= 0.0))
         return fail("ftr_time_seq: bad argument");
     hipStream_t s = (hipStream_t)stream;
-    for (int i = 0; i < warmup; ++i)
+    const auto t_begin = std::chrono::steady_clock::now();
+    auto expired = [&]() {
+        if (timeout_s <= 0.0) return false;
+        std::chrono::duration<double> d = std::chrono::steady_clock::now() - t_begin;
+        return d.count() > timeout_s;
+    };
+    for (int i = 0; i < warmup; ++i) {
         if (ftr_launch_seq(seqs + (size_t)(i % nsets) * n_per_iter, n_per_iter,
                            stream))
             return 1;
+        // a candidate far slower than expected shows while the warm-up is
+        // still being enqueued (the queue fills and launches block)
+        if ((i & 63) == 63 && expired()) {
+            fail("timed out after %.3f s (warm-up launch %d of %d)", timeout_s, i + 1, warmup);
+            return FTR_TIMEOUT;
+        }
+    }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     FTR_HIP(hipEventCreate(&e0));
     hipError_t e = hipEventCreate(&e1);
@@ -248,27 +264,77 @@ int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
         return fail("hipEventCreate: %s", hipGetErrorString(e));
     }
     int rc = 0;
+    bool late = false;
     float ms = 0.f;
     do {
         if ((e = hipEventRecord(e0, s)) != hipSuccess) break;
-        for (int i = 0; i < iters && !rc; ++i)
+        for (int i = 0; i < iters && !rc && !late; ++i) {
             rc = ftr_launch_seq(seqs + (size_t)(i % nsets) * n_per_iter,
                                 n_per_iter, stream);
-        if (rc) break;
+            if ((i & 63) == 63 && expired()) late = true;   // stop enqueueing, too
+        }
+        if (rc || late) break;
         if ((e = hipEventRecord(e1, s)) != hipSuccess) break;
-        if ((e = hipEventSynchronize(e1)) != hipSuccess) break;
+        if (timeout_s > 0.0) {
+            // wait with a deadline: poll the closing event instead of blocking on it. The work
+            // stays enqueued when the deadline passes (nothing can take it back); the caller
+            // treats the candidate as failed and drains the stream before the next one.
+            while ((e = hipEventQuery(e1)) == hipErrorNotReady) {
+                if (expired()) {
+                    late = true;
+                    break;
+                }
+                std::this_thread::sleep_for(std::chrono::microseconds(50));
+            }
+            if (late) {
+                (void)hipGetLastError();
+                e = hipSuccess;
+                break;
+            }
+            if (e != hipSuccess) break;
+        } else if ((e = hipEventSynchronize(e1)) != hipSuccess) {
+            break;
+        }
         e = hipEventElapsedTime(&ms, e0, e1);
     } while (0);
     if (rc) (void)hipStreamSynchronize(s);  // drain what was enqueued before failing
-    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e0);              // a pending event is released when it completes
     (void)hipEventDestroy(e1);
     if (rc) return 1;
+    if (late) {
+        fail("timed out after %.3f s (up to %d timed launches enqueued)", timeout_s, iters * n_per_iter);
+        return FTR_TIMEOUT;
+    }
     if (e != hipSuccess) {
         (void)hipGetLastError();
         return fail("timing failed: %s (%d)", hipGetErrorString(e), (int)e);
     }
     *ms_mean = ms / (float)iters;
     return 0;
+}
+
+int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
+                 int warmup, int iters, void *stream, float *ms_mean) {
+    return ftr_time_seq_deadline(seqs, n_per_iter, nsets, warmup, iters, stream, 0.0, ms_mean);
+}
+
+int ftr_stream_idle(void *stream, double timeout_s) {
+    const auto t_begin = std::chrono::steady_clock::now();
+    for (;;) {
+        hipError_t e = hipStreamQuery((hipStream_t)stream);
+        if (e == hipSuccess) return 0;
+        if (e != hipErrorNotReady) {
+            (void)hipGetLastError();
+            return fail("hipStreamQuery failed: %s (%d)", hipGetErrorString(e), (int)e);
+        }
+        std::chrono::duration<double> d = std::chrono::steady_clock::now() - t_begin;
+        if (d.count() > timeout_s) {
+            (void)hipGetLastError();
+            fail("stream still busy after %.3f s", timeout_s);
+            return FTR_TIMEOUT;
+        }
+        std::this_thread::sleep_for(std::chrono::microseconds(100));
+    }
 }
 
 int ftr_time(ftr_module_t mod, const unsigned grid[3], const unsigned block[3],

@@ -125,16 +125,14 @@ def run_default_schedule(ops, tensors, stream=0):
         K = op.reduce_axis[0].extent
         for b in range(nb):
             args = [rt.ptr(tensors[0][b]), rt.ptr(tensors[1][b]), rt.ptr(out[b]), i32(M), i32(N), i32(K),
-                    i32(1 if op.attrs.get("transposeB") else 0)]
+                    i32(1 if op.attrs.get("transposeB") else 0), i32(0)]
             _naive("gemm_f32_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
         return
     if op.kind == "gemm":
-        if op.attrs.get("transposeA"):
-            raise NotImplementedError("transposeA")
         M, N = [a.extent for a in op.axis]
         K = op.reduce_axis[0].extent
         args = [rt.ptr(tensors[0]), rt.ptr(tensors[1]), rt.ptr(out), i32(M), i32(N), i32(K),
-                i32(1 if op.attrs.get("transposeB") else 0)]
+                i32(1 if op.attrs.get("transposeB") else 0), i32(1 if op.attrs.get("transposeA") else 0)]
         _naive("gemm_f32_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
     elif op.kind == "gemm_int8":
         M, N = [a.extent for a in op.axis]
@@ -226,26 +224,53 @@ class Measurer(object):
         torch.cuda.synchronize()
         return ok, metric
 
-    def evaluate(self, plan, number=10, warmup=2, warm_ms=WARM_MS):
+    def evaluate(self, plan, number=10, warmup=2, warm_ms=WARM_MS, timeout=0.0):
         """ms per run of ``plan``; raises on build failure or wrong output.
         Candidates are compiled between measurements, so each one meets an
-        idle device: ``warm_ms`` of untimed runs bring the clocks up first."""
+        idle device: ``warm_ms`` of untimed runs bring the clocks up first.
+
+        ``timeout`` > 0 is the candidate's time limit in seconds
+        (flextensor/measure.py:63-74 gives a child process that long): every
+        wait on the device has that deadline and raises
+        ``runtime.DeviceTimeout`` when it passes. The work already enqueued
+        cannot be taken back, so the next candidate first waits (with its own
+        deadline) for the stream to run empty; while it has not, candidates
+        keep failing instead of being timed behind foreign work."""
         import torch
+        timeout = float(timeout or 0.0)
+        stream = current_stream()
+        if timeout > 0:
+            rt.stream_idle(stream, timeout)
+            for m in _abandoned:          # the stream is empty: what an overrun left loaded can go
+                m.close()
+            del _abandoned[:]
         built = plan.build()
         try:
             first = self.sets[0]
             first[-1].zero_()
             built(*first)
+            if timeout > 0:
+                rt.stream_idle(stream, timeout)
             torch.cuda.synchronize()
             ok, metric = self.check(first[-1])
             if not ok:
                 raise WrongResult("output differs from the default schedule (metric %g)" % metric)
-            return built.time(self.sets, warmup=warmup, iters=max(int(number), 1), warm_ms=warm_ms)
+            return built.time(self.sets, warmup=warmup, iters=max(int(number), 1), warm_ms=warm_ms,
+                              timeout=timeout)
         finally:
+            if timeout > 0:
+                # unloading a module waits for its kernels: give up after the limit and leave the
+                # modules to the garbage collector rather than block on a candidate that overran
+                try:
+                    rt.stream_idle(stream, timeout)
+                except rt.DeviceTimeout:
+                    _abandoned.extend(built.modules)
+                    built.modules = []
             built.close()
 
 
 _measurers = {}
+_abandoned = []       # modules of candidates that overran their time limit, kept loaded until the stream is idle
 
 
 def get_measurer(task_key, seed=0):
@@ -256,7 +281,7 @@ def get_measurer(task_key, seed=0):
     return _measurers[key]
 
 
-def build_and_eval(lib, s, bufs, target, dev_id, rpc_info=None, number=1):
+def build_and_eval(lib, s, bufs, target, dev_id, rpc_info=None, number=1, timeout=0.0):
     """Build plan ``s``, verify it, time ``number`` launches; returns mean ms.
 
     ``lib`` (a path the reference writes the exported library to) receives the
@@ -270,12 +295,12 @@ def build_and_eval(lib, s, bufs, target, dev_id, rpc_info=None, number=1):
         codes = s.compile()
         with open(lib, "wb") as f:
             f.write(codes[-1])
-    return get_measurer(s.task_key).evaluate(s, number=number)
+    return get_measurer(s.task_key).evaluate(s, number=number, timeout=timeout)
 
 
-def _evaluate(s, bufs, target, dev_id, number=1, q=None):
+def _evaluate(s, bufs, target, dev_id, number=1, q=None, timeout=0.0):
     """In-process build + time (flextensor/measure.py:29-52)."""
-    time_cost = build_and_eval(None, s, bufs, target, dev_id, None, number)
+    time_cost = build_and_eval(None, s, bufs, target, dev_id, None, number, timeout=timeout)
     if q:
         q.put(time_cost)
     return time_cost
@@ -290,15 +315,24 @@ def servant_routine(func, que, *args, **kwargs):
 
 
 def master_routine(timeout, func, *args, **kwargs):
-    """Run ``func`` and return its result, or the exception it raised.
+    """Run ``func`` and return its result, or the exception it raised
+    (a ``runtime.DeviceTimeout`` when the time limit passed).
 
     The reference runs ``func`` in a forked child and waits ``timeout`` seconds
     (flextensor/measure.py:63-74). A process that has initialised the GPU must
-    not fork, so the call is made in-process; kernels built from the templates
-    have compile-time loop bounds and always terminate.
+    not fork, so the call is made in-process and the limit is enforced where
+    the time goes: ``timeout`` is handed to ``func`` as its ``timeout``
+    keyword (``_evaluate`` / ``build_and_eval`` pass it to the device waits,
+    which poll with a deadline). Kernels built from the templates have
+    compile-time loop bounds and always terminate; a candidate that overruns
+    is abandoned, not killed.
     """
-    del timeout
     try:
+        if timeout:
+            import inspect
+            params = inspect.signature(func).parameters
+            if "timeout" in params or any(p.kind == p.VAR_KEYWORD for p in params.values()):
+                kwargs.setdefault("timeout", timeout)
         return func(*args, **kwargs)
     except Exception as e:  # noqa: BLE001
         return e

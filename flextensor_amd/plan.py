@@ -143,8 +143,10 @@ class BuiltPlan(object):
         else:
             rt.launch_seq(launches, stream=current_stream())
 
-    def time(self, tensor_sets, warmup=2, iters=10, warm_ms=0.0):
-        """Mean ms per run, rotating through ``tensor_sets``.
+    def time(self, tensor_sets, warmup=2, iters=10, warm_ms=0.0, timeout=0.0):
+        """Mean ms per run, rotating through ``tensor_sets``. ``timeout`` > 0
+        is a deadline in seconds for each wait on the device
+        (runtime.DeviceTimeout when it passes).
 
         ``warm_ms`` > 0 keeps the device busy with untimed runs for about that
         long first: after an idle period the clocks take on the order of
@@ -155,9 +157,9 @@ class BuiltPlan(object):
         sets = [self.launches(ts) for ts in tensor_sets]
         stream = current_stream()
         if warm_ms > 0:
-            probe = rt.time_seq(sets, warmup=1, iters=3, stream=stream)
+            probe = rt.time_seq(sets, warmup=1, iters=3, stream=stream, timeout=timeout)
             warmup = max(warmup, int(min(warm_ms / max(probe, 1e-4), 1e6)))
-        return rt.time_seq(sets, warmup=warmup, iters=iters, stream=stream)
+        return rt.time_seq(sets, warmup=warmup, iters=iters, stream=stream, timeout=timeout)
 
     def close(self):
         for m in self.modules:

@@ -21,18 +21,24 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libftrocm.so")
 CACHE_DIR = os.environ.get("FLEXTENSOR_AMD_KCACHE", os.path.join(_HERE, "_kcache"))
 DEFAULT_ARCH = "gfx950"
-ABI_VERSION = 1
+ABI_VERSION = 2
+FTR_TIMEOUT = 2
 
 EXPORTS = (
     "ftr_abi_version", "ftr_last_error", "ftr_compile_to_code", "ftr_code_free",
     "ftr_module_load", "ftr_compile", "ftr_module_free", "ftr_module_attrs",
     "ftr_launch", "ftr_launch_seq", "ftr_launch_seq_static_ws", "ftr_time", "ftr_time_seq",
+    "ftr_time_seq_deadline", "ftr_stream_idle",
     "ftr_device_props", "ftr_device_count",
 )
 
 
 class RuntimeError_(RuntimeError):
     """A failing call into libftrocm.so."""
+
+
+class DeviceTimeout(RuntimeError_):
+    """A call with a deadline gave up waiting; the device work is still enqueued."""
 
 
 class _Props(ctypes.Structure):
@@ -121,6 +127,10 @@ def lib():
         L.ftr_time_seq.argtypes = [
             ctypes.POINTER(_LaunchDesc), ctypes.c_int, ctypes.c_int, ctypes.c_int,
             ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
+        L.ftr_time_seq_deadline.argtypes = [
+            ctypes.POINTER(_LaunchDesc), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+            ctypes.c_int, ctypes.c_void_p, ctypes.c_double, ctypes.POINTER(ctypes.c_float)]
+        L.ftr_stream_idle.argtypes = [ctypes.c_void_p, ctypes.c_double]
         L.ftr_device_props.argtypes = [ctypes.c_int, ctypes.POINTER(_Props)]
         L.ftr_device_count.restype = ctypes.c_int
         if L.ftr_abi_version() != ABI_VERSION:
@@ -133,7 +143,8 @@ def lib():
 def _check(rc, what):
     if rc != 0:
         msg = lib().ftr_last_error()
-        raise RuntimeError_("%s: %s" % (what, msg.decode("utf-8", "replace") if msg else "?"))
+        text = "%s: %s" % (what, msg.decode("utf-8", "replace") if msg else "?")
+        raise DeviceTimeout(text) if rc == FTR_TIMEOUT else RuntimeError_(text)
 
 
 def device_count():
@@ -388,9 +399,15 @@ def launch_seq_static_ws(launches, binds, stream=0):
            "ftr_launch_seq_static_ws")
 
 
-def time_seq(sets, warmup=3, iters=20, stream=0):
+def stream_idle(stream=0, timeout=0.0):
+    """Wait up to ``timeout`` seconds for the stream to run empty; raises DeviceTimeout if it does not."""
+    _check(lib().ftr_stream_idle(ctypes.c_void_p(stream), float(timeout)), "ftr_stream_idle")
+
+
+def time_seq(sets, warmup=3, iters=20, stream=0, timeout=0.0):
     """Mean ms per iteration; ``sets`` is a list of equally long launch lists
-    (one per buffer set) that the timed loop rotates through."""
+    (one per buffer set) that the timed loop rotates through. ``timeout`` > 0
+    is a deadline in seconds for the whole call (DeviceTimeout when it passes)."""
     n_per = len(sets[0])
     flat = []
     for s in sets:
@@ -399,7 +416,7 @@ def time_seq(sets, warmup=3, iters=20, stream=0):
         flat.extend(s)
     arr = _desc_array(flat)
     ms = ctypes.c_float()
-    rc = lib().ftr_time_seq(arr, n_per, len(sets), int(warmup), int(iters),
-                            ctypes.c_void_p(stream), ctypes.byref(ms))
+    rc = lib().ftr_time_seq_deadline(arr, n_per, len(sets), int(warmup), int(iters),
+                                     ctypes.c_void_p(stream), float(timeout or 0.0), ctypes.byref(ms))
     _check(rc, "ftr_time_seq")
     return ms.value

@@ -282,17 +282,16 @@ class Scheduler(object):
         ops, _ = self.task.func(*self.task.args)
         op = flatten_graph(ops)[0][self.op_pos]
         candidates = []
+        # an operator the templates cannot seed (no admissible tile, a variant that is not built)
+        # simply starts from random points; any other error is a bug in the templates and surfaces
         try:
             candidates.extend(gfx950.seed_configs(op, limit=self.seed_limit))
-        except Exception:  # noqa: BLE001
+        except (gfx950.InvalidConfig, NotImplementedError):
             pass
-        try:
-            from .tuned import lookup
-            shipped = lookup(self.task_key, similar=True) if self.warm_start else None
-            if shipped is not None and self.op_pos < len(shipped.op_config_lst):
-                candidates.append(shipped.op_config_lst[self.op_pos])
-        except Exception:  # noqa: BLE001
-            pass
+        from .tuned import lookup
+        shipped = lookup(self.task_key, similar=True) if self.warm_start else None
+        if shipped is not None and self.op_pos < len(shipped.op_config_lst):
+            candidates.append(shipped.op_config_lst[self.op_pos])
         points = []
         for cfg in candidates:
             indices = {}
@@ -530,8 +529,8 @@ class Scheduler(object):
             cfg, op_pos = self._fetch_config(old_configs, config, mode)
             schedule_with_config(self.task_key, cfg, op_pos=op_pos, rewrite=self.rewrite)
             return True
-        except Exception:  # noqa: BLE001
-            return False
+        except (gfx950.InvalidConfig, NotImplementedError):
+            return False          # a point the templates refuse; anything else is a template bug and surfaces
 
     # ---- evaluation ----------------------------------------------------
     def _fetch_config(self, old_configs, config, mode):
@@ -560,8 +559,8 @@ class Scheduler(object):
             try:
                 s, _ = schedule_with_config(self.task_key, cfg, op_pos=op_pos, rewrite=self.rewrite)
                 plans.append(s)
-            except Exception:  # noqa: BLE001
-                plans.append(None)
+            except (gfx950.InvalidConfig, NotImplementedError):
+                plans.append(None)        # a point the templates refuse costs inf, as a failed build does
         if self._pool is None or self._pool.workers != self.parallel:
             if self._pool is not None:
                 self._pool.close()
@@ -576,8 +575,10 @@ class Scheduler(object):
             try:
                 if measurer is None:
                     measurer = get_measurer(self.task_key)
-                res.append(float(measurer.evaluate(plan, number=number)))
-            except Exception:  # noqa: BLE001
+                # the per-candidate time limit of the reference (timeout -> inf, scheduler.py:742-748):
+                # the device wait has a deadline; nothing is killed and no process is re-executed
+                res.append(float(measurer.evaluate(plan, number=number, timeout=self.timeout)))
+            except Exception:  # noqa: BLE001  (a failing candidate never propagates)
                 res.append(float("inf"))
         return res
 
@@ -717,14 +718,11 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
         # config (inline flags, special knobs) is the context instead, so that
         # the shipped point keeps its measured cost when it seeds the search.
         if kwargs.get("warm_start", True):
-            try:
-                from .tuned import lookup
-                shipped = lookup(task_key, similar=True)
-                if shipped is not None and shipped.graph_config and \
-                        len(shipped.graph_config.get("special") or []) == len(task.special_space):
-                    configs = Config([], dict(shipped.graph_config))
-            except Exception:  # noqa: BLE001
-                pass
+            from .tuned import lookup
+            shipped = lookup(task_key, similar=True)
+            if shipped is not None and shipped.graph_config and \
+                    len(shipped.graph_config.get("special") or []) == len(task.special_space):
+                configs = Config([], dict(shipped.graph_config))
 
     schedulers = []
     try:
@@ -890,5 +888,38 @@ def schedule_with_config_ops(ops, bufs, configs, op_pos=None, target="rocm", tas
 
 
 def schedule_ops_with_config(s, op_lst, configs, target):
-    raise RuntimeError("schedule_ops_with_config operates on TVM schedules; "
-                       "use schedule_with_config_ops")
+    """Schedule an already flattened operator list with given configs
+    (flextensor/scheduler.py:1189-1220): ``op_lst`` is in producer -> consumer
+    order and ``configs.op_config_lst[i]`` belongs to ``op_lst[i]``. The
+    reference mutates the TVM schedule ``s`` and returns it; here ``s`` is a
+    KernelPlan to refill (or None) and the lowered plan is returned. The
+    plan's buffers are the graph's placeholders in order of first use, then
+    the output of the last operator."""
+    if target not in SUPPORTED_TARGETS:
+        raise RuntimeError("Currently no support for target %s" % target)
+    op_lst = list(op_lst)
+    if not op_lst:
+        raise ValueError("empty operator list")
+    consumed = set()
+    for op in op_lst:
+        for t in op.input_tensors:
+            consumed.add(t.op)
+    outputs = [op for op in op_lst if op not in consumed]
+    if len(outputs) != 1:
+        raise ValueError("expected one output operator, found %d" % len(outputs))
+    order, _ = flatten_graph(outputs)
+    if order != op_lst:
+        raise ValueError("op_lst is not the flattened graph of its output operator "
+                         "(configs are matched to operators by position)")
+    inputs = []
+    for op in op_lst:
+        for t in op.input_tensors:
+            if not isinstance(t.op, ComputeOp) and t not in inputs:
+                inputs.append(t)
+    bufs = inputs + [outputs[0].output(0)]
+    plan, _ = schedule_with_config_ops(outputs, bufs, configs, target=target,
+                                       task_key=getattr(s, "task_key", None))
+    if isinstance(s, KernelPlan):
+        s.__dict__.update(plan.__dict__)
+        return s
+    return plan

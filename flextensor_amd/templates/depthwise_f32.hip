@@ -56,6 +56,7 @@
 #define CQ FT_CQ
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 #define PLANES (CB * CC * FACT)
 #define TILES_H ((CP + TH - 1) / TH)
@@ -165,6 +166,18 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     }
 }
 #else
+/* Every global access of the direct kernel is a raw buffer access: an
+ * element that must read as zero (padding row or column, idle lane) or must
+ * not be written gets an offset beyond the buffer, for which a load returns 0
+ * and a store is dropped by the hardware. Nothing branches, so the row loads
+ * of a patch are all issued back to back and their round trips overlap. */
+#define OOB 0x80000000u
+#define X_BYTES (CB * CC * CH * CW * 4)
+#define W_BYTES (CC * FACT * CR * CS * 4)
+#define O_BYTES (CB * CC * FACT * CP * CQ * 4)
+#define LD_AUX (NT_LOAD ? 2 : 0)     /* bit 1 of the cache policy operand: non-temporal */
+#define ST_AUX (NT_STORE ? 2 : 0)
+
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                    float* __restrict__ O)
@@ -176,8 +189,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     const bool live = (lane < LPW) && (gid < ITEMS);
 #else
     const int gid = blockIdx.x * NT + threadIdx.x;
-    if (gid >= ITEMS) return;
-    const bool live = true;
+    const bool live = gid < ITEMS;
 #endif
     const int tw = gid % TILES_W;
     const int th = (gid / TILES_W) % TILES_H;
@@ -185,16 +197,31 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     const int b = plane / (CC * FACT);
     const int co = plane % (CC * FACT);
     const int ci = co / FACT;
-    const float* x = X + (size_t)(live ? (b * CC + ci) : 0) * (CH * CW);
-    const float* wp = Wt + (size_t)(live ? co : 0) * (CR * CS);
-    float* o = O + (size_t)plane * (CP * CQ);
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(Wt), 0, W_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, O_BYTES, 0x00020000);
+    const int xplane = (b * CC + ci) * (CH * CW);      /* first element of the input plane */
+    const int oplane = plane * (CP * CQ);
 
     float wreg[CR][CS];
+    {
+        /* the kernel's CR*CS taps: 128-bit loads (dword-aligned is enough for buffer loads) and a tail */
+        const unsigned wo = live ? (unsigned)(co * (CR * CS)) * 4u : OOB;
+        float wflat[(CR * CS + 3) / 4 * 4];
 #pragma unroll
-    for (int r = 0; r < CR; ++r)
+        for (int t = 0; t + 4 <= CR * CS; t += 4) {
+            const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, (int)wo, t * 4, 0));
+            wflat[t] = v[0]; wflat[t + 1] = v[1]; wflat[t + 2] = v[2]; wflat[t + 3] = v[3];
+        }
 #pragma unroll
-        for (int s = 0; s < CS; ++s)
-            wreg[r][s] = wp[r * CS + s];
+        for (int t = (CR * CS) / 4 * 4; t < CR * CS; ++t)
+            wflat[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rw, (int)wo, t * 4, 0));
+#pragma unroll
+        for (int r = 0; r < CR; ++r)
+#pragma unroll
+            for (int s = 0; s < CS; ++s)
+                wreg[r][s] = wflat[r * CS + s];
+    }
 
     const int oh0 = th * TH;
     const int ow0 = tw * TW;
@@ -208,17 +235,57 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         for (int j = 0; j < TW; ++j)
             acc[i][j] = 0.0f;
 
+    auto store_row = [&](int i) {
+        const int oh = oh0 + i;
+        const bool row_ok = live && (CP % TH == 0 || oh < CP);
+#if VEC_OUT
+        f32x4 v;
+        v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
+        const unsigned vo = row_ok ? (unsigned)(oplane + oh * CQ + ow0) * 4u : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ro, (int)vo, 0, ST_AUX);
+#else
 #pragma unroll
-    for (int y = 0; y < IH_T; ++y) {
+        for (int j = 0; j < TW; ++j) {
+            const bool ok = row_ok && (CQ % TW == 0 || ow0 + j < CQ);
+            const unsigned vo = ok ? (unsigned)(oplane + oh * CQ + ow0 + j) * 4u : OOB;
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc[i][j]), ro, (int)vo, 0, ST_AUX);
+        }
+#endif
+    };
+    /* one element of input row ih (any int), column iw (any int); zero outside the image */
+    auto load1 = [&](int ih, int iw) -> float {
+        const bool ok = live && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+        const unsigned vo = ok ? (unsigned)(xplane + ih * CW + iw) * 4u : OOB;
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)vo, 0, LD_AUX));
+    };
+#if (SHFL || VEC_IN)
+    /* the four centre columns of input row ih0 + y */
+    auto load_row4 = [&](int y) -> f32x4 {
         const int ih = ih0 + y;
         const bool row_ok = live && (unsigned)ih < (unsigned)CH;
-        const float* xr = x + ih * CW;
+        const unsigned vo = row_ok ? (unsigned)(xplane + ih * CW + ow0) * 4u : OOB;
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo, 0, LD_AUX));
+    };
+    f32x4 rows[IH_T];
+#pragma unroll
+    for (int y = 0; y < IH_T; ++y) rows[y] = load_row4(y);
+#if !SHFL
+    /* the halo columns left and right of the centre vector */
+    float halo[IH_T][IW_T];
+#pragma unroll
+    for (int y = 0; y < IH_T; ++y)
+#pragma unroll
+        for (int j = 0; j < IW_T; ++j)
+            if (j < PAD || j >= PAD + 4) halo[y][j] = load1(ih0 + y, iw0 + j);
+#endif
+#endif
+
+#pragma unroll
+    for (int y = 0; y < IH_T; ++y) {
         float in[IW_T];
 #if SHFL
         {
-            f32x4 v = (f32x4)(0.0f);
-            if (row_ok) v = NT_LOAD ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + ow0))
-                                   : *reinterpret_cast<const f32x4*>(xr + ow0);
+            const f32x4 v = rows[y];
             /* column ow0-1 is the last column of the lane below, column ow0+4
              * the first column of the lane above; image borders read zero */
             const float v0 = v[0], v3 = v[3];
@@ -230,25 +297,14 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         }
 #elif VEC_IN
         {
-            f32x4 v = (f32x4)(0.0f);
-            if (row_ok) v = NT_LOAD ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xr + ow0))
-                                   : *reinterpret_cast<const f32x4*>(xr + ow0);
+            const f32x4 v = rows[y];
 #pragma unroll
-            for (int j = 0; j < IW_T; ++j) {
-                if (j >= PAD && j < PAD + 4) {
-                    in[j] = v[(j - PAD) & 3];
-                } else {
-                    const int iw = iw0 + j;
-                    in[j] = (row_ok && (unsigned)iw < (unsigned)CW) ? xr[iw] : 0.0f;
-                }
-            }
+            for (int j = 0; j < IW_T; ++j)
+                in[j] = (j >= PAD && j < PAD + 4) ? v[(j - PAD) & 3] : halo[y][j];
         }
 #else
 #pragma unroll
-        for (int j = 0; j < IW_T; ++j) {
-            const int iw = iw0 + j;
-            in[j] = (row_ok && (unsigned)iw < (unsigned)CW) ? xr[iw] : 0.0f;
-        }
+        for (int j = 0; j < IW_T; ++j) in[j] = load1(ih0 + y, iw0 + j);
 #endif
         /* input row y feeds output row i through tap r when y == i*STR + r*DIL */
 #pragma unroll
@@ -265,26 +321,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
             }
         }
     }
-
-    if (!live) return;
+    /* stores last: vector memory operations retire in issue order, so a load
+     * issued behind a store would have to wait for the store's round trip */
 #pragma unroll
-    for (int i = 0; i < TH; ++i) {
-        const int oh = oh0 + i;
-        if (CP % TH != 0 && oh >= CP) continue;
-        float* orow = o + oh * CQ + ow0;
-#if VEC_OUT
-        f32x4 v;
-        v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
-#if NT_STORE
-        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(orow));
-#else
-        *reinterpret_cast<f32x4*>(orow) = v;
-#endif
-#else
-#pragma unroll
-        for (int j = 0; j < TW; ++j)
-            if (CQ % TW == 0 || ow0 + j < CQ) orow[j] = acc[i][j];
-#endif
-    }
+    for (int i = 0; i < TH; ++i) store_row(i);
 }
 #endif

@@ -29,6 +29,14 @@
 //               lds modifier, 16 bytes per lane): no staging registers, no
 //               LDS store instructions; the row swizzle is applied on the
 //               global side, since a wavefront's 64 chunks land contiguously
+//               DTL 3: the same data path with the instruction order of the
+//               main loop written out and pinned: the LDS fragment reads of
+//               the next k-step and the direct-to-LDS loads of the tile after
+//               next are issued one at a time between the MFMAs of the current
+//               k-step, and the one barrier of a tile sits a quarter into its
+//               last k-step, so that the matrix cores always have queued work
+//               (left to itself the compiler issues the fragment reads right
+//               before their first use and waits for them)
 //   NT_STORE    1: non-temporal stores for C
 //   CVEC        1: the MFMA operands are swapped (the core computes the
 //               transposed tile), so a lane holds four consecutive columns of
@@ -131,6 +139,9 @@ typedef i32x4 acc_t;
 #if DTL
 #if PAD > 0 || STAGES != 2 || A_CHUNKS % NT != 0 || B_CHUNKS % NT != 0
 #error "direct-to-LDS tiles need unpadded rows, two buffers and whole rounds of chunks"
+#endif
+#if DTL == 3 && ((BK / MFMA_K) % 2 != 0 || REP_M * REP_N / 4 + REP_M + REP_N > REP_M * REP_N || REP_M * REP_N / 4 + EA + EB > REP_M * REP_N)
+#error "the pinned schedule needs an even number of k-steps per tile and enough MFMAs per k-step to interleave with"
 #endif
 typedef __attribute__((address_space(3))) void lds_void;
 #endif
@@ -308,9 +319,90 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             }
         };
         dma_tile(0, 0);
+#if DTL != 3
         __builtin_amdgcn_s_waitcnt(0x0F70);     /* vmcnt(0): this wavefront's chunks are in LDS */
         __syncthreads();
-#if DTL == 2
+#endif
+#if DTL == 3
+        /* Pinned schedule. Two fragment sets alternate by k-step parity (an even
+         * number of k-steps per tile, so a tile ends on the set it began with and
+         * nothing is copied). Slot m is what is issued before MFMA m of a k-step:
+         *   not the last k-step:  fragment read m of the next k-step   (m < NR)
+         *   last k-step:          at m == NB the wait for tile kt+1 and the barrier
+         *                         (everybody has read the last fragments of tile kt
+         *                         one k-step ago), then fragment read m - NB of tile
+         *                         kt+1 and direct-to-LDS load m - NB of tile kt+2,
+         *                         which goes into the buffer the barrier has freed
+         *                         and has a whole tile period to land. */
+#define NKS (BK / MFMA_K)
+#define NM (REP_M * REP_N)
+#define NR (REP_M + REP_N)
+#define NB (NM / 4)
+        const int arow = wm * REP_M * MFMA + li;
+        const int brow = wn * REP_N * MFMA + li;
+        i32x4 fA[2][REP_M], fB[2][REP_N];
+        auto rd = [&](int buf, int kk, int set, int g) {
+            if (g < REP_M)
+                fA[set][g] = *reinterpret_cast<const i32x4*>(&As[buf][(arow + g * MFMA) * SROW + PCOL(arow + g * MFMA, kk + 16 * lg)]);
+            else
+                fB[set][g - REP_M] = *reinterpret_cast<const i32x4*>(&Bs[buf][(brow + (g - REP_M) * MFMA) * SROW + PCOL(brow + (g - REP_M) * MFMA, kk + 16 * lg)]);
+        };
+        auto dma_one = [&](int kt, int buf, int e) {
+            const int k0 = kt * BK;
+            if (e < EA) {
+                unsigned vo = a_voff[e];
+                if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+                dma16(ra, &As[buf][(e * NT + wv * 64) * 16], vo, k0);
+            } else {
+                unsigned vo = b_voff[e - EA];
+                if (KP != K) vo = (k0 + b_col[e - EA] < K) ? vo : OOB;
+                dma16(rb, &Bs[buf][((e - EA) * NT + wv * 64) * 16], vo, k0);
+            }
+        };
+        /* one tile; NEXT: tile kt+1 exists (its fragments are fetched), NEXT2: tile kt+2 exists */
+#define I8_TILE(NEXT, NEXT2)                                                                          \
+        _Pragma("unroll")                                                                             \
+        for (int ks = 0; ks < NKS; ++ks) {                                                            \
+            const int set = ks & 1;                                                                   \
+            _Pragma("unroll")                                                                         \
+            for (int m = 0; m < NM; ++m) {                                                            \
+                if (ks + 1 < NKS) {                                                                   \
+                    if (m < NR) rd(cur, (ks + 1) * MFMA_K, set ^ 1, m);                               \
+                } else if (NEXT) {                                                                    \
+                    if (m == NB) {                                                                    \
+                        __builtin_amdgcn_s_waitcnt(0x0F70);                                           \
+                        __syncthreads();                                                              \
+                    }                                                                                 \
+                    if (m >= NB && m - NB < NR) rd(cur ^ 1, 0, set ^ 1, m - NB);                      \
+                    if ((NEXT2) && m >= NB && m - NB < EA + EB) dma_one(kt + 2, cur, m - NB);         \
+                }                                                                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                    \
+                acc[m / REP_N][m % REP_N] = MFMA_OP(fA[set][m / REP_N], fB[set][m % REP_N], acc[m / REP_N][m % REP_N]); \
+                __builtin_amdgcn_sched_barrier(0);                                                    \
+            }                                                                                         \
+        }
+        if (KT > 1) dma_tile(1, 1);
+        /* tile 0 has landed when at most the loads of tile 1 are outstanding */
+        if (KT > 1) __builtin_amdgcn_s_waitcnt(0x0F70 | ((EA + EB) & 15) | (((EA + EB) >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < NR; ++g) rd(0, 0, 0, g);
+        int kt = 0;
+        for (; kt + 2 < KT; ++kt) {
+            const int cur = kt & 1;
+            I8_TILE(1, 1)
+        }
+        for (; kt + 1 < KT; ++kt) {
+            const int cur = kt & 1;
+            I8_TILE(1, 0)
+        }
+        {
+            const int cur = kt & 1;
+            I8_TILE(0, 0)
+        }
+#undef I8_TILE
+#elif DTL == 2
         /* with fragment prefetch: the LDS reads of step t+1 are issued before
          * the MFMAs of step t, across the tile boundary as well */
         const int arow = wm * REP_M * MFMA + li;

@@ -94,9 +94,9 @@ class GemmView(object):
         self.kind = kind
         self.conv = None
         self.groups = 1
+        self.trans_a = False
         if kind == "gemm":
-            if op.attrs.get("transposeA"):
-                raise NotImplementedError("transposeA is not on the tuned path")
+            self.trans_a = bool(op.attrs.get("transposeA"))     # A stored [K][M] (ops.py:1093-1100)
             self.M, self.N = op.axis[0].extent, op.axis[1].extent
             self.K = op.reduce_axis[0].extent
             self.mode = 2 if op.attrs.get("transposeB") else 0
@@ -176,7 +176,7 @@ I8_BK = (64, 128, 256)
 def _gemm_space(view):
     space = Space()
     i8 = view.dtype == "int8"
-    reps = (1, 2, 3, 4, 6, 8)
+    reps = (1, 2, 3, 4, 5, 6, 7, 8)
     space.add_subspace("split_m_0", TileSplitSpace(view.M, reps=reps), "spatial")
     space.add_subspace("split_n_1", TileSplitSpace(view.N, reps=reps), "spatial")
     bks = I8_BK if i8 else F32_BK
@@ -194,7 +194,8 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7], explicit=True), "unroll")
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7, 8] if i8 else [1, 2, 3, 4, 5, 6, 7], explicit=True),
+                       "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
     space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
@@ -244,9 +245,11 @@ SPECIAL_DEFAULTS = {
 # depth 5 = two stages with the fragment-prefetch pipeline (int8 GEMM)
 # depth -> (LDS buffers, global prefetch distance); 5 = int8: MFMA fragment prefetch, fp32: tiles
 # loaded straight into LDS; int8 only:
-# 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch;
+# 6 = tiles loaded straight into LDS (no staging registers), 7 = 6 with MFMA fragment prefetch,
+# 8 = 7 with the main loop's instruction order written out (fragment reads and tile loads issued
+# one at a time between the MFMAs);
 # fp32: 6 and 7 = 5 with three and four LDS buffers (two and three tiles requested ahead)
-PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7: (2, 1)}
+PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7: (2, 1), 8: (2, 1)}
 
 
 def special_knobs(kind):
@@ -293,7 +296,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE:
+    if depth not in PIPELINE or (depth == 8 and view.dtype != "int8"):
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
     if view.dtype != "int8" and depth >= 6:
@@ -345,6 +348,11 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         if depth >= 6:
             if pad > 0 or (bm * bk // 16) % nt or (bn * bk // 16) % nt:
                 raise InvalidConfig("direct-to-LDS tiles need unpadded rows and whole rounds of 16-byte chunks")
+            if depth == 8:
+                nm, nr, loads = rm * rn, rm + rn, (bm + bn) * bk // 16 // nt
+                if (bk // mfma_k) % 2 or nm // 4 + nr > nm or nm // 4 + loads > nm:
+                    raise InvalidConfig("the written-out schedule needs an even number of k-steps per tile "
+                                        "and enough MFMAs per k-step to interleave with")
         elif (ceil_div(bm * bk // 16, nt) + ceil_div(bn * bk // 16, nt)) * 4 * pd > 160:
             raise InvalidConfig("global->LDS staging needs too many registers")
         lds = stages * (bm + bn) * (bk + max(pad, 0))
@@ -374,6 +382,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     if apad < -1 or (apad >= 0 and apad % 4 != 0) or bpad % 4 != 0:
         raise InvalidConfig("fp32 LDS padding must keep 16-byte alignment")
     av = 4 if view.K % 4 == 0 else 1
+    if view.trans_a:
+        av = 4 if view.M % 4 == 0 else 1      # vectors run along M, the contiguous axis of a [K][M] operand
     if view.mode == 0:
         bv = 4 if view.N % 4 == 0 else 1
     elif view.mode == 2:
@@ -381,6 +391,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     else:
         bv = 1
     dtl = depth >= 5          # fp32: tiles loaded straight into LDS
+    if dtl and view.trans_a:
+        raise InvalidConfig("a transposed A operand is transposed in registers: register-staged pipelines only")
     if dtl:
         if view.mode == 0 and view.N % 4 == 0 and bn % 64 == 0 and (bpad_auto or bpad == 0):
             bv, bpad = 4, 0   # B in 16-byte chunks too: unpadded rows, columns swizzled by k
@@ -392,8 +404,14 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
             raise InvalidConfig("direct-to-LDS tiles need 16-byte A chunks in whole wavefronts and unpadded A rows")
         if view.mode == 2 and (bv != 4 or (bn * bk // 4) % 64):
             raise InvalidConfig("direct-to-LDS tiles need 16-byte B chunks in whole wavefronts")
-        if view.mode != 2 and bn % 64 and not (64 % bn == 0 and bpad == 0 and (bn * bk) % 64 == 0):
-            raise InvalidConfig("direct-to-LDS tiles need BN % 64 == 0, or BN dividing 64 with unpadded B rows")
+        if view.mode != 2 and bv == 1 and bn % 64:
+            # B one float per lane: a wavefront writes 64 consecutive floats, so rows that are
+            # not multiples of 64 floats land unpadded, in whole wavefronts per tile
+            if bpad_auto:
+                bpad = 0
+            if bpad != 0 or (bn * bk) % 64:
+                raise InvalidConfig("direct-to-LDS tiles with rows that are not multiples of 64 floats need "
+                                    "unpadded B rows and whole wavefronts of floats per tile")
     if apad < 0 and (bk & (bk - 1)) != 0:
         apad = 4              # the chunk swizzle needs a power-of-two row
     sa = bk + max(apad, 0)
@@ -427,6 +445,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     if max(a_bytes, b_bytes, view.groups * view.M * view.N * 4) >= 2 ** 31:
         raise InvalidConfig("operands of 2 GiB or more are not addressable by the buffer loads")
     D.update(MODE=view.mode, SPLITK=splitk, WAVES_K=waves_k, APAD=apad, BPAD=bpad, AV=av, BV=bv, PD=pd)
+    if view.trans_a:
+        D.update(TA=1)
     if dtl:
         D.update(DTL=1)
     specs = []
@@ -505,8 +525,12 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         h, w, pad = h + 2 * pad, w + 2 * pad, 0
     ih_t = (th - 1) * a["stride"][0] + (r_ext - 1) * a["dilation"][0] + 1
     iw_t = (tw - 1) * a["stride"][0] + (s_ext - 1) * a["dilation"][0] + 1
-    if th * tw + iw_t + r_ext * s_ext > 200:
+    # the 128-bit input path requests every row of the patch before the first is used
+    vec_rows = (tw == 4 and a["stride"][0] == 1 and w % 4 == 0 and q == w and pad + 4 <= iw_t)
+    if th * tw + (ih_t * iw_t if vec_rows else iw_t) + r_ext * s_ext > 200:
         raise InvalidConfig("lane patch needs too many registers")
+    if max(b * c * h * w, b * cout * p * q) * 4 >= 2 ** 31:
+        raise InvalidConfig("tensors of 2 GiB or more are not addressable by the buffer accesses")
     nt = waves * 64
     items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
     ldsp = int(_special(special, "lds_planes")[0])
@@ -537,7 +561,6 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=shfl,
              CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=a["stride"][0], PAD=pad,
              DIL=a["dilation"][0], FACT=a["factor"], CP=p, CQ=q)
-    del ih_t
     return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
                        (nt, 1, 1),
                        [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]

@@ -8,6 +8,10 @@
 //   MODE 2  dense GEMM, B^T   A row-major [M][K], B stored [N][K]
 //                             (the transposeB branch, ops.py:1101-1104)
 //           MODE 0 and 2 also run a batch of CG such GEMMs (ops.py:1111-1158)
+//           TA 1 (MODE 0 and 2): A is stored [K][M] (the transposeA branches,
+//           ops.py:1093-1100). Its tile is fetched in vectors along M and
+//           transposed on the way into LDS, where it has the usual [BM][BK]
+//           layout; register-staged pipelines only.
 //   MODE 1  conv2d NCHW       A = weight [Kout][C*R*S], B = im2col gather of
 //                             the input with zero padding folded into the
 //                             load predicate, N = batch*OH*OW
@@ -104,6 +108,11 @@
 #else
 #define COLOUT 0
 #endif
+#ifdef FT_TA
+#define TA FT_TA
+#else
+#define TA 0
+#endif
 #ifdef FT_SK_PER
 #define SK_PER FT_SK_PER
 #else
@@ -189,9 +198,17 @@ typedef f32x4 acc_t;
 #error "BK must be a multiple of 4*(64/MFMA)"
 #endif
 
-/* ---- A tile: BM x BK, vectors of AV floats along K ---------------------- */
+/* ---- A tile: BM x BK, vectors of AV floats along K (along M when A is stored [K][M]) */
+#if TA
+#if MODE == 1 || DTL
+#error "a transposed A operand: dense GEMM modes, register-staged pipelines"
+#endif
+#define A_CHUNKS_ROW (BM / AV)
+#define A_CHUNKS (BK * A_CHUNKS_ROW)
+#else
 #define A_CHUNKS_ROW (BK / AV)
 #define A_CHUNKS (BM * A_CHUNKS_ROW)
+#endif
 #define EA ((A_CHUNKS + NT - 1) / NT)
 /* ---- B tile: BK x BN, vectors of BV floats along N (along K in MODE 2) --- */
 #if MODE == 2
@@ -231,8 +248,33 @@ typedef f32x4 acc_t;
 #else
 #define BSWK(k) ((((k) >> 2) & 1) << 3)     /* 32 floats per lane group */
 #endif
-#elif BV != 1 || !(BN % 64 == 0 || (64 % BN == 0 && BPAD == 0))
-#error "direct-to-LDS tiles: B goes one float per lane; a wavefront covers part of one row, or whole unpadded rows"
+#elif BV != 1 || !(BN % 64 == 0 || BPAD == 0)
+#error "direct-to-LDS tiles: B goes one float per lane; a wavefront covers part of one padded row, or 64 floats of the unpadded tile"
+#endif
+#if BV == 1 && BPAD == 0 && (BN % 64 == 0 || BN == 32 || BN == 16)
+/* B one float per lane into unpadded rows: the four (two) k rows that the lane
+ * groups of an MFMA read together would sit in the same banks. Every lane
+ * computes its own global address, so any permutation of the tile is free on
+ * the global side: the element of logical (k, n), k-group g = (k >> 2) & (KG-1),
+ * lives at row (k & ~3) | ((k & 3) ^ BSW_R(g)), column n ^ BSW_C(g). Both only
+ * move an element inside the 64 floats one wavefront writes, and they send the
+ * lane groups of one MFMA operand read to disjoint banks:
+ *   rows of 64 floats or more  columns XOR-ed by g * MFMA
+ *   rows of 32 floats          16x16x4: column bit 4 by g's low bit, row parity
+ *                              by g's high bit; 32x32x2: row parity by g
+ *   rows of 16 floats          the row's low two bits by g */
+#define BSWZ1 1
+#define KG (64 / MFMA)
+#if BN % 64 == 0
+#define BSW_R(g) 0
+#define BSW_C(g) ((g) * MFMA)
+#elif BN == 32 && MFMA == 16
+#define BSW_R(g) ((g) >> 1)
+#define BSW_C(g) (((g) & 1) << 4)
+#else
+#define BSW_R(g) (g)
+#define BSW_C(g) 0
+#endif
 #endif
 #endif
 typedef __attribute__((address_space(3))) void lds_void;
@@ -376,6 +418,12 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         b_col[e] = ACOL(b_row[e], (q % B_CHUNKS_ROW) * BV);
 #elif defined(BSWZ)
         b_col[e] = ((q % B_CHUNKS_ROW) ^ BSWK(b_row[e])) * BV;
+#elif defined(BSWZ1)
+        {   /* float q of the tile is physical (row, column): fetch the logical element that lives there */
+            const int pr = q / BN, g = (pr >> 2) & (KG - 1);
+            b_row[e] = (pr & ~3) | ((pr & 3) ^ BSW_R(g));
+            b_col[e] = (q % BN) ^ BSW_C(g);
+        }
 #else
         b_col[e] = (q % B_CHUNKS_ROW) * BV;
 #endif
@@ -560,10 +608,18 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     unsigned a_voff[EA], b_voff[EB];
 #pragma unroll
     for (int e = 0; e < EA; ++e) {
+#if TA
+        /* a_row = k inside the tile, a_col = first of AV consecutive rows m (M % AV == 0) */
+        const int m = m0 + a_col[e];
+        bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
+        if (M % BM != 0) ok = ok && (m < M);
+        a_voff[e] = ok ? (unsigned)((gi * K + a_row[e]) * M + m) * 4u : OOB;
+#else
         const int m = m0 + a_row[e];
         bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
         if (M % BM != 0) ok = ok && (m < M);
         a_voff[e] = ok ? (unsigned)((gi * M + m) * K + a_col[e]) * 4u : OOB;
+#endif
     }
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
@@ -596,8 +652,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
             unsigned vo = a_voff[e];
+#if TA
+            if (KP != K) vo = (k0 + a_row[e] < K) ? vo : OOB;
+            areg[set][e] = LOAD_A(rsrc_a, vo, k0 * (M * 4));
+#else
             if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
             areg[set][e] = LOAD_A(rsrc_a, vo, k0 * 4);
+#endif
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
@@ -630,8 +691,20 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     auto store_lds = [&](int buf, int set) {
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
-            if ((A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS))
+            if ((A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS)) {
+#if TA
+                /* transpose: element i of the vector is row a_col + i, column k = a_row */
+#if AV == 4
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    As[buf][(a_col[e] + i) * SA + ACOL(a_col[e] + i, a_row[e])] = areg[set][e][i];
+#else
+                As[buf][a_col[e] * SA + ACOL(a_col[e], a_row[e])] = areg[set][e];
+#endif
+#else
                 *reinterpret_cast<avec_t*>(&As[buf][a_row[e] * SA + ACOL(a_row[e], a_col[e])]) = areg[set][e];
+#endif
+            }
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
@@ -663,6 +736,16 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
         for (int j = 0; j < REP_N; ++j)
             bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ (MFMA == 16 ? (lg << 4) : (lg << 5));
+#elif defined(BSWZ1)
+        /* logical (kb + 4*lg + s, n) sits at row kb + 4*lg + (s ^ BSW_R(lg)), column n ^ BSW_C(lg) */
+        const float* bs = &Bs[buf][(4 * lg) * SB];
+        int bcolx[REP_N], browx[4];
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j)
+            bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ BSW_C(lg);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            browx[s] = (s ^ BSW_R(lg)) * SB;
 #else
         const float* bs = &Bs[buf][(4 * lg) * SB + wn * REP_N * MFMA + li];
 #endif
@@ -687,6 +770,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                     b[j] = b4[j][s];
 #elif defined(BSWZ)
                     b[j] = bs[(kb + s) * SB + (bcolx[j] ^ (MFMA == 16 ? 0 : (((kb >> 2) & 1) << 5)))];
+#elif defined(BSWZ1)
+                    b[j] = bs[kb * SB + browx[s] + bcolx[j]];
 #else
                     b[j] = bs[(kb + s) * SB + j * MFMA];
 #endif

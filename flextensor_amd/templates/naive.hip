@@ -13,17 +13,16 @@
 
 extern "C" __global__ __launch_bounds__(256)
 void gemm_f32_naive(const float* __restrict__ A, const float* __restrict__ B,
-                    float* __restrict__ C, int M, int N, int K, int transB)
+                    float* __restrict__ C, int M, int N, int K, int transB, int transA)
 {
+    /* A is [M][K], or [K][M] when transA; B is [K][N], or [N][K] when transB */
     const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (long long)M * N) return;
     const int i = (int)(gid / N), j = (int)(gid % N);
+    const size_t a0 = transA ? (size_t)i : (size_t)i * K, as = transA ? (size_t)M : 1;
+    const size_t b0 = transB ? (size_t)j * K : (size_t)j, bs = transB ? 1 : (size_t)N;
     float acc = 0.0f;
-    if (transB) {
-        for (int k = 0; k < K; ++k) acc += A[(size_t)i * K + k] * B[(size_t)j * K + k];
-    } else {
-        for (int k = 0; k < K; ++k) acc += A[(size_t)i * K + k] * B[(size_t)k * N + j];
-    }
+    for (int k = 0; k < K; ++k) acc += A[a0 + k * as] * B[b0 + k * bs];
     C[gid] = acc;
 }
 

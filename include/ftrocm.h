@@ -25,7 +25,10 @@
 extern "C" {
 #endif
 
-#define FTR_ABI_VERSION 1
+#define FTR_ABI_VERSION 2
+
+/* Return code of the calls that take a deadline when it passes. */
+#define FTR_TIMEOUT 2
 
 typedef struct ftr_module *ftr_module_t;
 
@@ -121,6 +124,22 @@ int ftr_time(ftr_module_t mod, const unsigned grid[3], const unsigned block[3],
  * kernel's traffic in HBM rather than in the last-level cache. */
 int ftr_time_seq(const ftr_launch_desc_t *seqs, int n_per_iter, int nsets,
                  int warmup, int iters, void *stream, float *ms_mean);
+
+/* ftr_time_seq with a deadline of `timeout_s` seconds (0 = none) over the
+ * whole call: the closing event is polled instead of waited for, and when the
+ * deadline passes the call returns FTR_TIMEOUT with the work still enqueued
+ * (device work cannot be taken back; no process is killed). Stands in for the
+ * time limit the reference puts on a candidate by running it in a child
+ * process that the parent gives `timeout` seconds
+ * (flextensor/measure.py:63-74, flextensor/scheduler.py:742-748). */
+int ftr_time_seq_deadline(const ftr_launch_desc_t *seqs, int n_per_iter,
+                          int nsets, int warmup, int iters, void *stream,
+                          double timeout_s, float *ms_mean);
+
+/* Wait up to `timeout_s` seconds for `stream` to run empty: 0 when it is
+ * idle, FTR_TIMEOUT when work is still pending. What a caller does after a
+ * timed-out candidate before it measures the next one. */
+int ftr_stream_idle(void *stream, double timeout_s);
 
 /* Bytes of the static device workspace ftr_launch_seq_static_ws binds. */
 #define FTR_STATIC_WS_BYTES (64u << 20)

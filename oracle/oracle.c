@@ -18,7 +18,7 @@
  *   ft_conv2d_nchw       flextensor/nn/ops.py:419-479  (reduce order rc, rw, rh;
  *                        reads the materialised padded tensor, as the graph does)
  *   ft_depthwise_nchw    flextensor/nn/ops.py:622-678  (reduce order rw, rh)
- *   ft_gemm_f32          flextensor/nn/ops.py:1074-1108 (transposeB optional)
+ *   ft_gemm_f32          flextensor/nn/ops.py:1074-1108 (all four transposeA / transposeB branches)
  *   ft_gemm_i8           flextensor/test/test_tvm/legacy/gemm_int8.py:15-21
  *
  * Pinning (see tests/test_oracle.py): every function is checked against
@@ -140,17 +140,17 @@ int ft_depthwise_nchw(const float *X, const float *Wt, float *O, int NB, int C, 
 
 /* C[i][j] = sum_k A[i][k] * B[k][j]  (transB: B stored [N][K], B[j][k]) */
 void ft_gemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int transB,
-                 int fma)
+                 int fma, int transA)
 {
+    /* A is [M][K], or [K][M] when transA; B is [K][N], or [N][K] when transB (ops.py:1093-1108) */
     for (int i = 0; i < M; ++i)
         for (int j = 0; j < N; ++j) {
             float acc = 0.0f;
-            if (transB)
-                for (int k = 0; k < K; ++k)
-                    acc = mac(acc, A[(size_t)i * K + k], B[(size_t)j * K + k], fma);
-            else
-                for (int k = 0; k < K; ++k)
-                    acc = mac(acc, A[(size_t)i * K + k], B[(size_t)k * N + j], fma);
+            for (int k = 0; k < K; ++k) {
+                const float a = transA ? A[(size_t)k * M + i] : A[(size_t)i * K + k];
+                const float b = transB ? B[(size_t)j * K + k] : B[(size_t)k * N + j];
+                acc = mac(acc, a, b, fma);
+            }
             C[(size_t)i * N + j] = acc;
         }
 }

@@ -117,14 +117,15 @@ def depthwise_nchw_c(x, wt, stride=1, padding=0, dilation=1, fma=True):
     return out
 
 
-def gemm_f32_c(a, b, transB=False, fma=True):
+def gemm_f32_c(a, b, transB=False, fma=True, transA=False):
     a, ap = _f32(a)
     b, bp = _f32(b)
-    m, k = a.shape
+    k, m = a.shape if transA else a.shape[::-1]
     n = b.shape[0] if transB else b.shape[1]
     assert (b.shape[1] if transB else b.shape[0]) == k
     out = np.empty((m, n), dtype=np.float32)
-    lib().ft_gemm_f32(ap, bp, out.ctypes.data_as(_f32p), m, n, k, int(bool(transB)), int(fma))
+    lib().ft_gemm_f32(ap, bp, out.ctypes.data_as(_f32p), m, n, k, int(bool(transB)), int(fma),
+                      int(bool(transA)))
     return out
 
 

@@ -33,7 +33,7 @@ def _compile_only(monkeypatch):
         return
     from flextensor_amd import plan as plan_mod
 
-    def compile_and_skip(self, plan):
+    def compile_and_skip(self, plan, **kwargs):
         plan.compile()
         pytest.skip("kernels compiled")
 

@@ -112,6 +112,31 @@ def test_raw_cabi_launch_and_timing():
         mod.launch((0,), (256,), args)
 
 
+def test_time_limit_abandons_an_overrunning_measurement_and_recovers():
+    """The per-candidate time limit (flextensor/measure.py:63-74): a measurement that cannot
+    finish inside it comes back as DeviceTimeout (-> inf for the search) without anything being
+    killed; once the stream has drained the same plan measures normally and is still right."""
+    import time
+    register(gemm, "gemm", "gemm", (512, 512, 512), "rocm", 0)
+    key = key_of("gemm", "gemm", (512, 512, 512))
+    s, bufs = schedule_with_config(key, Config([], None))
+    m = Measurer(key, seed=2)
+    t0 = time.time()
+    with pytest.raises(rt.DeviceTimeout):
+        # ten million timed launches of a kernel of a few microseconds cannot fit into 0.2 s
+        m.evaluate(s, number=10 ** 7, warmup=0, warm_ms=0.0, timeout=0.2)
+    assert time.time() - t0 < 20
+    rt.stream_idle(current_stream(), 120.0)           # every enqueued kernel finishes by itself
+    ms = m.evaluate(s, number=20, timeout=30.0)
+    assert 0 < ms < 5
+    from flextensor_amd.measure import master_routine, _evaluate
+    slow = master_routine(0.2, m.evaluate, s, number=10 ** 7, warmup=0, warm_ms=0.0)
+    assert isinstance(slow, rt.DeviceTimeout)
+    rt.stream_idle(current_stream(), 120.0)
+    fine = master_routine(30.0, _evaluate, s, bufs, "rocm", 0, number=5)
+    assert isinstance(fine, float) and 0 < fine < 5
+
+
 # ------------------------------------------------------- golden fixtures --
 
 def test_golden_gemm_small_ragged():
@@ -308,6 +333,14 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16, st=6), [-1, 8]),
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=72, st=6), [0, 0]),
     ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=32, st=7, ks=1), [-1, 0]),
+    # unpadded B rows permuted against bank conflicts: every row width / MFMA shape of the permutation
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=16, st=5), [-1, 0]),    # 32 floats, 16x16x4
+    ((2, 16, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=4, rn=1, mf=16, bk=16, st=5), [-1, 0]),    # 64 floats, 16x16x4
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=2, mf=32, bk=16, st=5), [-1, 0]),    # 128 floats, 32x32x2
+    ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16, st=5), [-1, 0]),     # 16 floats, stride 2, K tail
+    # rows that neither divide nor are multiples of 64 floats: the tile lands flat, not permuted
+    ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=5, mf=16, bk=32, st=5), [-1, 0]),      # 80 floats, N=392
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=3, mf=16, bk=16, st=5), [0, 0]),     # 48 floats
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)
@@ -493,6 +526,41 @@ def test_gemm_transpose_b_vs_oracle(oracle):
         assert rel(out, oracle.gemm_f32_c(a, b, transB=True)) <= TOL
 
 
+def test_gemm_transpose_a_vs_oracle(oracle):
+    """The transposeA branches (flextensor/nn/ops.py:1093-1100): A stored [K][M], with B stored
+    either way; ragged M (vector and scalar transposing loads), split K, default config."""
+    for (M, K, N), tb in (((160, 96, 224), False), ((160, 96, 224), True), ((50, 72, 90), False),
+                          ((37, 64, 29), True)):
+        def wrap(M, K, N, tb=tb):
+            A = placeholder((K, M), name="A")
+            B = placeholder((N, K) if tb else (K, N), name="B")
+            C = op_gemm(A, B, transposeA=True, transposeB=tb)
+            return [C.op], [A, B, C]
+        name = "gemm_t%s" % ("t" if tb else "n")
+        register(wrap, "gemm", name, (M, K, N), "rocm", 0)
+        key = key_of("gemm", name, (M, K, N))
+        ops, bufs = wrap(M, K, N)
+        assert bufs[-1].shape == (M, N)
+        a, b = seeded_inputs(bufs, seed=M + K)
+        ref = oracle.gemm_f32_c(a, b, transA=True, transB=tb)
+        assert rel(ref, a.astype(np.float64).T @ (b.astype(np.float64).T if tb else b.astype(np.float64))) < 1e-5
+        kp = ceil_div(K, 16) * 16
+        cfgs = [None, gcfg(M, N, kp, 2, 1, 2, 1, 16, 16, st=3), gcfg(M, N, kp, 1, 2, 1, 1, 32, 16, st=1)]
+        if kp % 48 == 0:
+            cfgs.append(gcfg(M, N, kp, 1, 2, 2, 2, 16, 16, sk=3, st=2))
+        for cfg in cfgs:
+            out = run_plan(key, Config([cfg] if cfg else [], None), [a, b])
+            assert rel(out, ref) <= TOL, (M, K, N, tb, cfg)
+        with pytest.raises(Exception):      # tiles straight into LDS cannot transpose
+            schedule_with_config(key, Config([gcfg(M, N, kp, 2, 1, 2, 1, 16, 16, st=5)], None))
+        # and the default-schedule kernel the search checks candidates against
+        dev = [torch.from_numpy(x).cuda() for x in (a, b)]
+        out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+        run_default_schedule(ops, dev + [out], stream=current_stream())
+        torch.cuda.synchronize()
+        assert rel(out.cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("M,K,N,kn", [
     (256, 256, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=64)),
     (256, 512, 384, dict(wm=1, rm=4, wn=2, rn=2, mf=16, bk=128, st=1)),
@@ -509,6 +577,11 @@ def test_gemm_transpose_b_vs_oracle(oracle):
     (200, 336, 136, dict(wm=2, rm=2, wn=1, rn=4, mf=16, bk=64, st=7)),       # same, ragged, one step per tile
     (256, 64, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=64, st=7)),        # same, a single tile
     (512, 1024, 512, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=256, st=7)),     # same, 16 wavefronts, four steps per tile
+    (512, 512, 512, dict(wm=2, rm=4, wn=2, rn=4, mf=16, bk=128, st=8)),      # written-out instruction order, four tiles
+    (200, 336, 136, dict(wm=2, rm=4, wn=1, rn=4, mf=16, bk=128, st=8)),      # same, ragged M and N, K tail, three tiles
+    (256, 128, 256, dict(wm=2, rm=4, wn=2, rn=4, mf=16, bk=128, st=8)),      # same, a single tile
+    (256, 256, 256, dict(wm=2, rm=4, wn=2, rn=4, mf=16, bk=128, st=8)),      # same, two tiles
+    (512, 512, 256, dict(wm=2, rm=2, wn=2, rn=4, mf=32, bk=64, st=8)),       # same, 32x32x32, two k-steps per tile
 ])
 def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
     _gemm_int8_case(oracle, M, K, N, kn, None)
@@ -533,7 +606,7 @@ def _gemm_int8_case(oracle, M, K, N, kn, store):
     a, b = seeded_inputs(bufs, seed=K)
     assert a.min() == -128 and a.max() == 127
     g = None
-    if store is not None or kn.get("st") in (6, 7):       # direct-to-LDS tiles need the swizzled (unpadded) layout
+    if store is not None or kn.get("st") in (6, 7, 8):       # direct-to-LDS tiles need the swizzled (unpadded) layout
         g = {k: [] for k in KEYS}
         g["inline"], g["special"] = [[0]], [[-1, 0], [store or 0]]
     out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], g), [a, b])

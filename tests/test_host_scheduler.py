@@ -421,3 +421,27 @@ def test_seed_points_cover_the_decisive_knobs_and_belong_to_the_space():
     # plenty of tiles: no K split
     _, _, seeds = seeds_of(I8)
     assert all(c["reduce"][0][0] == 1 for c in seeds)
+
+
+def test_schedule_ops_with_config_takes_a_flattened_op_list():
+    """flextensor/scheduler.py:1189-1220: configs are matched to the operators of an already
+    flattened list by position; the plan comes back (a plan passed in is refilled)."""
+    from flextensor_amd.scheduler import schedule_ops_with_config
+    key = "conv2d_baseline0_(1, 64, 56, 56, 64, 3, 1, 1, 1, 1)_rocm(0)"
+    task = TASK_TABLE[key]
+    ops, bufs = task.func(*task.args)
+    op_lst, _ = flatten_graph(ops)
+    assert [op.kind for op in op_lst] == ["zero_pad2d", "conv2d_nchw"]
+    ref, _ = schedule_with_config(key, Config([], None))
+    plan = schedule_ops_with_config(None, op_lst, Config([], None), "rocm")
+    assert [sp.defines for sp in plan.specs] == [sp.defines for sp in ref.specs]
+    assert [tuple(b.shape) for b in plan.bufs] == [tuple(b.shape) for b in bufs]
+    # a graph config that materialises the padding gives two kernels; an existing plan is refilled
+    g = {k: [] for k in gfx950.Space.valid_type_keys}
+    g["inline"] = [[0, 0]]
+    again = schedule_ops_with_config(plan, op_lst, Config([], g), "rocm")
+    assert again is plan and [sp.kernel for sp in plan.specs] == ["zero_pad2d_f32", "igemm_f32"]
+    with pytest.raises(ValueError):
+        schedule_ops_with_config(None, list(reversed(op_lst)), Config([], None), "rocm")
+    with pytest.raises(RuntimeError):
+        schedule_ops_with_config(None, op_lst, Config([], None), "cuda")

@@ -187,6 +187,14 @@ def test_gemm_f32(oracle, gold):
     assert rel(oracle.gemm_f32_c(a, b), gold["gemm_c"]) < 1e-6
     assert rel(oracle.gemm_f32_c(a, b, fma=False), gold["gemm_c"]) < 1e-6
     assert rel(oracle.gemm_f32_c(a, np.ascontiguousarray(b.T), transB=True), gold["gemm_c"]) < 1e-6
+    # the transposeA branches (flextensor/nn/ops.py:1093-1100): A stored [K][M]; a transposed
+    # or mixed-up operand would not reproduce the same product from the same data
+    at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
+    assert np.array_equal(oracle.gemm_f32_c(at, b, transA=True), oracle.gemm_f32_c(a, b))
+    assert np.array_equal(oracle.gemm_f32_c(at, bt, transA=True, transB=True), oracle.gemm_f32_c(a, b))
+    r = np.random.default_rng(5)
+    x, y = r.uniform(-1, 1, (7, 5)).astype(np.float32), r.uniform(-1, 1, (7, 3)).astype(np.float32)
+    assert rel(oracle.gemm_f32_c(x, y, transA=True), x.astype(np.float64).T @ y.astype(np.float64)) < 1e-6
     assert rel(oracle.gemm_np(a, b), gold["gemm_c"]) < 1e-13
     # identity and a permutation matrix: exact
     eye = np.eye(64, dtype=np.float32)

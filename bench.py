@@ -4,10 +4,12 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-headline]
                     [--workload NAME]
 
-One step = one run of the tuned kernel plan of the headline workload
-(conv2d NCHW fp32, N=1, C=64, H=W=56, K=64, 3x3, stride 1, pad 1) over
-seeded synthetic inputs that are resident in HBM before the timed region.
-W untimed steps, then exactly K steps between two device synchronisations.
+One step = one run of the tuned kernel plan of the headline workload, the
+largest single-GPU configuration of the benchmark set (int8 x int8 -> int32
+GEMM, M = N = K = 4096, B stored K-major), over seeded synthetic inputs that
+are resident in HBM before the timed region. The device is first kept busy
+for about 150 ms (idle clocks need that long to settle), then W untimed
+steps, then exactly K steps between two device synchronisations.
 Prints ONE JSON line with the whole-job throughput (`value`, TFLOP/s), the
 roofline position of the dominant kernel measured with HIP events on the
 launch stream, the same figures for the other benchmark configurations
@@ -43,31 +45,52 @@ WORKLOADS = [
      57802752, 25708544, "hbm", "f32"),
     ("gemm_i8_4096", "gemm_gemm_int8_(4096, 4096, 4096)_rocm(0)", 2 * 4096 ** 3, 100663296, "mfma", "i8"),
 ]
-HEADLINE = 1  # configs[1] of BASELINE.json
+# The metric is quoted per operator, on no single configuration, so the headline is the largest
+# configuration that fits one GPU: configs[4] of the benchmark set (137 GOP per step).
+HEADLINE = 5
+HEADLINE_NOTE = " (largest single-GPU configuration, BASELINE.json configs[4])"
 
 
-def measured_traffic(name):
-    """HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE /
-    WRITE_SIZE runs of the shipped tuned config scaled by a plain copy of known
-    size (flextensor_amd/tuned/hbm_traffic.json); None when not recorded."""
+def config_hash(plan):
+    """Identifies the kernels a plan launches (templates' constants and geometry)."""
+    import hashlib
+    h = hashlib.sha256()
+    for spec in plan.specs:
+        h.update(("%s|%s|%s|%s;" % (spec.kernel, sorted(spec.defines.items()), spec.grid, spec.block)).encode())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(name, plan):
+    """(HBM bytes per launch of the plan's kernels, provenance) from rocprofv3
+    FETCH_SIZE / WRITE_SIZE runs scaled by a plain copy of known size
+    (flextensor_amd/tuned/hbm_traffic.json). The record carries the hash of
+    the kernels it was taken on: when the shipped config has changed since,
+    the figure is withheld (None) instead of being reported for other kernels."""
     path = os.path.join(ROOT, "flextensor_amd", "tuned", "hbm_traffic.json")
     try:
         with open(path) as f:
-            return json.load(f)[name]["hbm_bytes_per_launch"]
-    except Exception:  # noqa: BLE001
-        return None
+            rec = json.load(f)[name]
+    except (OSError, KeyError, ValueError):
+        return None, None
+    prov = {"measured": rec.get("measured"), "config_hash": rec.get("config_hash"),
+            "current_config_hash": config_hash(plan)}
+    if rec.get("config_hash") != prov["current_config_hash"]:
+        prov["stale"] = True
+        return None, prov
+    return rec["hbm_bytes_per_launch"], prov
 
 
-def roofline(name, bound, dtype, ops, nbytes, ms):
+def roofline(name, bound, dtype, ops, nbytes, ms, plan):
+    traffic, prov = measured_traffic(name, plan)
     if bound == "hbm":
         achieved = nbytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBS, "traffic": measured_traffic(name)}
+                "frac": achieved / PEAK_HBM_GBS, "traffic": traffic, "traffic_provenance": prov}
     peak = PEAK_I8_TOPS if dtype == "i8" else PEAK_F32_TFLOPS
     achieved = ops / (ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": peak,
             "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak,
-            "traffic": measured_traffic(name)}
+            "traffic": traffic, "traffic_provenance": prov}
 
 
 def gpu_workload(key, seed=0):
@@ -138,6 +161,8 @@ def copy_yardstick(mib, iters):
 
 def cpu_baseline_for(name, key, ops, budget_s):
     """Time the multi-threaded CPU port on the same seeded workload.
+    GEMM and convolution first run a small sweep over the port's register
+    tiles (and the GEMM's K tile), one pass each, and the best one is timed.
     Returns (ms per pass, threads, sample description)."""
     import numpy as np
     from flextensor_amd.measure import seeded_inputs
@@ -148,9 +173,21 @@ def cpu_baseline_for(name, key, ops, budget_s):
     host = seeded_inputs(bufs, 0)
     threads = o.baseline_threads()
     frac = 1.0
+    swept = ""
+
+    def once(f):
+        f()
+        t = time.perf_counter()
+        f()
+        return time.perf_counter() - t
+
     if name.startswith("gemm_f32"):
         out = np.empty(bufs[-1].shape, np.float32)
-        fn = lambda: o.baseline_gemm_f32(host[0], host[1], out, 256)  # noqa: E731
+        cands = [(v, tk) for v in range(len(o.baseline_gemm_f32_tiles())) for tk in (128, 256, 512)]
+        best = min(cands, key=lambda c: once(lambda: o.baseline_gemm_f32_v(host[0], host[1], out, c[1], c[0])))
+        swept = "; best of %d tilings: register tile %dx%d, K tile %d" % (
+            (len(cands),) + o.baseline_gemm_f32_tiles()[best[0]] + (best[1],))
+        fn = lambda: o.baseline_gemm_f32_v(host[0], host[1], out, best[1], best[0])  # noqa: E731
     elif name.startswith("gemm_i8"):
         out = np.zeros(bufs[-1].shape, np.int32)
         rows = 256
@@ -160,7 +197,12 @@ def cpu_baseline_for(name, key, ops, budget_s):
         a = task.args
         out = np.empty(bufs[-1].shape, np.float32)
         scratch = np.empty((a[0], a[1], a[2] + 2 * a[7], a[3] + 2 * a[7]), np.float32)
-        fn = lambda: o.baseline_conv2d(host[0], host[1], out, scratch, a[6], a[7], a[8])  # noqa: E731
+        cands = list(range(len(o.baseline_conv2d_tiles())))
+        best = min(cands, key=lambda v: once(lambda: o.baseline_conv2d_v(host[0], host[1], out, scratch,
+                                                                         a[6], a[7], a[8], v)))
+        swept = "; best of %d register tiles: %d output channels x %d columns" % (
+            (len(cands),) + o.baseline_conv2d_tiles()[best])
+        fn = lambda: o.baseline_conv2d_v(host[0], host[1], out, scratch, a[6], a[7], a[8], best)  # noqa: E731
     else:
         a = task.args
         out = np.empty(bufs[-1].shape, np.float32)
@@ -178,7 +220,18 @@ def cpu_baseline_for(name, key, ops, budget_s):
     ms = el / n * 1e3 / frac
     sample = "%d passes of the full workload" % n if frac == 1.0 else \
         "%d passes over the first %d output rows, scaled to the full matrix" % (n, rows)
-    return ms, threads, sample
+    return ms, threads, sample + swept
+
+
+def cpu_baseline_dict(name, key, ops, dtype, budget_s):
+    """The cpu_baseline object of one workload."""
+    ms, threads, sample = cpu_baseline_for(name, key, ops, budget_s)
+    naive_ms, naive_sample = cpu_naive_for(name, key)
+    return {"value": ops / (ms * 1e-3) / 1e12, "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "cores": threads,
+            "kind": "port", "ms": ms, "sample": sample + " (oracle/cpu_baseline.c, the "
+            "reference's llvm template structure in C/OpenMP; TVM itself is unavailable)",
+            "naive_1thread_ms": naive_ms, "naive_sample": naive_sample + " (oracle/oracle.c, the "
+            "default-schedule loop nest on one thread)"}
 
 
 def cpu_naive_for(name, key):
@@ -224,7 +277,7 @@ def main():
                     help="instead of a workload, run a plain device copy of this many MiB "
                          "(bandwidth yardstick; calibrates FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--workload", default=None, choices=[w[0] for w in WORKLOADS],
-                    help="time this configuration as the headline instead of configs[1] "
+                    help="time this configuration as the headline instead of the largest one "
                          "(used to profile one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -256,6 +309,9 @@ def main():
             args.steps = int(min(max(TIMED_WINDOW_MS / probe, 100), 100000))
         if args.warmup is None:
             args.warmup = int(min(max(WARM_MS / probe, 100), 100000))
+    # clocks first: ~150 ms of untimed runs whatever W is, so that the timed steps (and the event
+    # timing below) see the steady state and agree with each other
+    built.time(m.sets, warmup=1, iters=2, warm_ms=WARM_MS)
     if args.warmup > 0:
         wseq = launches * args.warmup
         rt._check(rt.lib().ftr_launch_seq(rt._desc_array(wseq), len(wseq), ctypes.c_void_p(stream)),
@@ -273,7 +329,7 @@ def main():
     if not ok:
         raise RuntimeError("headline plan fails the correctness gate (metric %g)" % metric)
     k_ms, _ = kernel_ms(built, m)
-    roof = roofline(name, bound, dtype, ops, nbytes, k_ms)
+    roof = roofline(name, bound, dtype, ops, nbytes, k_ms, plan)
     roof["kernel"] = plan.specs[-1].kernel
     roof["kernel_ms"] = k_ms
     # 24 000 launches of an empty kernel: left out of the short runs that a profiler wraps
@@ -286,7 +342,7 @@ def main():
         for (wname, wkey, wops, wbytes, wbound, wdtype) in WORKLOADS:
             b, mm, pl = gpu_workload(wkey)
             ms, met = kernel_ms(b, mm)
-            r = roofline(wname, wbound, wdtype, wops, wbytes, ms)
+            r = roofline(wname, wbound, wdtype, wops, wbytes, ms, pl)
             entry = {"workload": wname, "ms": ms, "dtype": wdtype,
                      "throughput": wops / (ms * 1e-3) / 1e12,
                      "throughput_unit": "TOP/s" if wdtype == "i8" else "TFLOP/s",
@@ -298,28 +354,17 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        ms, threads, sample = cpu_baseline_for(name, key, ops, args.cpu_seconds)
-        naive_ms, naive_sample = cpu_naive_for(name, key)
-        cpu = {"value": ops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "cores": threads,
-               "kind": "port", "ms": ms, "sample": sample + " (oracle/cpu_baseline.c, the "
-               "reference's llvm template structure in C/OpenMP; TVM itself is unavailable)",
-               "naive_1thread_ms": naive_ms, "naive_sample": naive_sample + " (oracle/oracle.c, the "
-               "default-schedule loop nest on one thread)"}
-        if not args.only_headline:
-            for entry, (wname, wkey, wops, _, _, _) in zip(per_config, WORKLOADS):
-                if wname == name:
-                    entry["cpu_ms"], entry["cpu_cores"], entry["cpu_naive_1thread_ms"] = ms, threads, naive_ms
-                    continue
-                cms, cth, _ = cpu_baseline_for(wname, wkey, wops, 1.0)
-                entry["cpu_ms"], entry["cpu_cores"] = cms, cth
-                entry["cpu_naive_1thread_ms"] = cpu_naive_for(wname, wkey)[0]
+        cpu = cpu_baseline_dict(name, key, ops, dtype, args.cpu_seconds)
+        for entry, (wname, wkey, wops, _, _, wdtype) in zip(per_config, WORKLOADS):
+            # every configuration carries its own baseline object; the headline's is the long sample
+            entry["cpu_baseline"] = cpu if wname == name else cpu_baseline_dict(wname, wkey, wops, wdtype, 1.0)
 
     line = {
         "metric": "best-config TFLOPS + % of MI355X roofline per op vs CPU llvm baseline",
         "value": value, "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name + (" (BASELINE.json configs[1])" if headline == HEADLINE else ""), "task_key": key,
+        "config": {"workload": name + (HEADLINE_NOTE if headline == HEADLINE else ""), "task_key": key,
                    "tuned_config": json.loads(json.dumps(plan.configs)),
                    "device": props["name"], "arch": props["arch"]},
         "roofline": roof, "cpu_baseline": cpu, "per_config": per_config,

@@ -361,9 +361,27 @@ class WalkerGroup(object):
                 walker.load_or_create_model(self.model_dir)
 
     def dump_data(self):
+        """Append what the search measured to the files of ``model_dir``: the
+        (points, costs) batches for the performance model and every walker's
+        transitions (model.py:469-474); the offline trainer reads them back."""
         if self.model_dir is not None:
+            self.dump_performance_data(os.path.join(self.model_dir, self.data_path))
             for walker in self.walkers.values():
                 walker.dump_data(self.model_dir)
+
+    def prepare_performance_data(self):
+        """Load the dumped (points, costs) batches of this group (model.py:458-467)."""
+        if self.model_dir is None:
+            raise RuntimeError("no model directory to read performance data from")
+        path = os.path.join(self.model_dir, self.data_path)
+        if os.path.exists(path):
+            self.load_performance_data(path)
+
+    def load_walker_data(self):
+        for walker in self.walkers.values():
+            walker.enable_learning()
+            if self.model_dir is not None and os.path.exists(os.path.join(self.model_dir, walker.data_path)):
+                walker.load_data(self.model_dir)
 
     # ---- performance model (use_model=True) ------------------------------
     def _perf_model(self):

@@ -76,6 +76,8 @@ def init_arg_parser(parser):
     parser.add_argument("--port", type=int, default=9190)
     parser.add_argument("--check", action="store_true")
     parser.add_argument("--number", help="launches per timing", type=int, default=50)
+    parser.add_argument("--perf_path", help="directory for the search's measured data and the learned models "
+                        "(read by python -m flextensor_amd.train and by --use_model)", type=str, default="")
     parser.add_argument("--warm_up", help="warm-up epochs x points, e.g. 4x16", type=str, default="")
     parser.add_argument("--shapes", help="shape table to tune (driver specific)", type=str,
                         default="baseline")
@@ -109,6 +111,9 @@ def run_driver(args, shapes, make_task, describe):
         kwargs["warm_up"] = (int(a), int(b))
     if getattr(args, "cold", False):
         kwargs["warm_start"] = False
+    if getattr(args, "perf_path", ""):
+        os.makedirs(args.perf_path, exist_ok=True)
+        kwargs["perf_path"] = args.perf_path
     try:
         for i, shape in enumerate(shapes[args.from_:end]):
             print("Optimize %s shape %s [%.6f]" % (describe, str(shape), time.time()), flush=True)

@@ -336,6 +336,8 @@ class Scheduler(object):
         for trial in range(self.trial):
             self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
         self._finish_with_model(configs, use_model)
+        self.walker_group.dump_data()
+        self.walker_group.clear_data()
         return self.walker_group.to_config(self.walker_group.top1())
 
     # ---- learned walk ---------------------------------------------------
@@ -507,8 +509,11 @@ class Scheduler(object):
                 for indices, result in zip(indices_lst, results):
                     if result < float("inf"):
                         self.walker_group.record(indices, result, random_reject=False)
+                self.walker_group.dump_data()        # keep what was measured for the offline trainer
                 self.walker_group.clear_data()
             self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
+        self.walker_group.dump_data()
+        self.walker_group.clear_data()
         if use_model:
             if minimal[1] < float("inf"):
                 self.walker_group.record(minimal[0], minimal[1], random_reject=False)

@@ -32,43 +32,73 @@ int ftb_num_threads(void)
 #endif
 }
 
-#define TI 6   /* register tile rows (unrolled)      */
-#define TJ 32  /* register tile columns (vectorised) */
+/* C[M][N] = A[M][K] * B[K][N]; register tile TI rows (unrolled) x TJ columns
+ * (vectorised), tk = K tile kept in cache. One function per register tile of
+ * the small sweep the benchmark runs (the reference's tuner would pick among
+ * such splits, flextensor/templates/cpu.py:330-372). */
+#define FTB_DEFINE_GEMM(TI, TJ)                                                                   \
+    static void gemm_f32_##TI##x##TJ(const float *A, const float *B, float *C, int M, int N,      \
+                                     int K, int tk)                                               \
+    {                                                                                             \
+        const int nio = (M + TI - 1) / TI, njo = (N + TJ - 1) / TJ;                               \
+        if (tk < 1) tk = K;                                                                       \
+        _Pragma("omp parallel for schedule(static)")                                              \
+        for (int t = 0; t < nio * njo; ++t) {                                                     \
+            const int i0 = (t / njo) * TI, j0 = (t % njo) * TJ;                                   \
+            const int ni = (M - i0) < TI ? (M - i0) : TI;                                         \
+            const int nj = (N - j0) < TJ ? (N - j0) : TJ;                                         \
+            float acc[TI][TJ];                                                                    \
+            memset(acc, 0, sizeof acc);                                                           \
+            for (int k0 = 0; k0 < K; k0 += tk) {                                                  \
+                const int k1 = (k0 + tk) < K ? (k0 + tk) : K;                                     \
+                if (ni == TI && nj == TJ) {                                                       \
+                    for (int k = k0; k < k1; ++k)                                                 \
+                        for (int i = 0; i < TI; ++i) {                                            \
+                            const float a = A[(size_t)(i0 + i) * K + k];                          \
+                            _Pragma("omp simd")                                                   \
+                            for (int j = 0; j < TJ; ++j)                                          \
+                                acc[i][j] += a * B[(size_t)k * N + j0 + j];                       \
+                        }                                                                         \
+                } else {                                                                          \
+                    for (int k = k0; k < k1; ++k)                                                 \
+                        for (int i = 0; i < ni; ++i) {                                            \
+                            const float a = A[(size_t)(i0 + i) * K + k];                          \
+                            for (int j = 0; j < nj; ++j)                                          \
+                                acc[i][j] += a * B[(size_t)k * N + j0 + j];                       \
+                        }                                                                         \
+                }                                                                                 \
+            }                                                                                     \
+            for (int i = 0; i < ni; ++i)                                                          \
+                for (int j = 0; j < nj; ++j) C[(size_t)(i0 + i) * N + j0 + j] = acc[i][j];        \
+        }                                                                                         \
+    }
+FTB_DEFINE_GEMM(6, 32)
+FTB_DEFINE_GEMM(4, 32)
+FTB_DEFINE_GEMM(8, 16)
+FTB_DEFINE_GEMM(6, 16)
+FTB_DEFINE_GEMM(4, 64)
 
-/* C[M][N] = A[M][K] * B[K][N]; tk = K tile kept in cache */
+/* number of register-tile variants, their (rows, columns), and the call by variant index */
+int ftb_gemm_f32_variants(void) { return 5; }
+void ftb_gemm_f32_variant_tile(int v, int *ti, int *tj)
+{
+    static const int t[5][2] = {{6, 32}, {4, 32}, {8, 16}, {6, 16}, {4, 64}};
+    *ti = t[v][0];
+    *tj = t[v][1];
+}
+void ftb_gemm_f32_v(const float *A, const float *B, float *C, int M, int N, int K, int tk, int v)
+{
+    switch (v) {
+    case 1: gemm_f32_4x32(A, B, C, M, N, K, tk); break;
+    case 2: gemm_f32_8x16(A, B, C, M, N, K, tk); break;
+    case 3: gemm_f32_6x16(A, B, C, M, N, K, tk); break;
+    case 4: gemm_f32_4x64(A, B, C, M, N, K, tk); break;
+    default: gemm_f32_6x32(A, B, C, M, N, K, tk); break;
+    }
+}
 void ftb_gemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int tk)
 {
-    const int nio = (M + TI - 1) / TI, njo = (N + TJ - 1) / TJ;
-    if (tk < 1) tk = K;
-#pragma omp parallel for schedule(static)
-    for (int t = 0; t < nio * njo; ++t) {
-        const int i0 = (t / njo) * TI, j0 = (t % njo) * TJ;
-        const int ni = (M - i0) < TI ? (M - i0) : TI;
-        const int nj = (N - j0) < TJ ? (N - j0) : TJ;
-        float acc[TI][TJ];
-        memset(acc, 0, sizeof acc);
-        for (int k0 = 0; k0 < K; k0 += tk) {
-            const int k1 = (k0 + tk) < K ? (k0 + tk) : K;
-            if (ni == TI && nj == TJ) {
-                for (int k = k0; k < k1; ++k)
-                    for (int i = 0; i < TI; ++i) {
-                        const float a = A[(size_t)(i0 + i) * K + k];
-#pragma omp simd
-                        for (int j = 0; j < TJ; ++j)
-                            acc[i][j] += a * B[(size_t)k * N + j0 + j];
-                    }
-            } else {
-                for (int k = k0; k < k1; ++k)
-                    for (int i = 0; i < ni; ++i) {
-                        const float a = A[(size_t)(i0 + i) * K + k];
-                        for (int j = 0; j < nj; ++j)
-                            acc[i][j] += a * B[(size_t)k * N + j0 + j];
-                    }
-            }
-        }
-        for (int i = 0; i < ni; ++i)
-            for (int j = 0; j < nj; ++j) C[(size_t)(i0 + i) * N + j0 + j] = acc[i][j];
-    }
+    gemm_f32_6x32(A, B, C, M, N, K, tk);
 }
 
 /* C[M][N] int32 = A[M][K] int8 * B[N][K]^T int8 */
@@ -102,53 +132,83 @@ static void pad2d(const float *X, float *P, int planes, int H, int W, int ph, in
     }
 }
 
-#define TKO 4  /* output channels per register tile (unrolled) */
-#define TW 16  /* output columns per register tile (vectorised) */
-
-/* conv2d NCHW, groups = 1. `scratch` holds the padded input
+/* conv2d NCHW, groups = 1; register tile TKO output channels (unrolled) x TW
+ * output columns (vectorised). `scratch` holds the padded input
  * (NB*C*(H+2ph)*(W+2pw) floats) and is written inside the call, as the
  * reference's two-operator graph does. */
+#define FTB_DEFINE_CONV(TKO, TW)                                                                  \
+    static void conv2d_nchw_##TKO##x##TW(const float *X, const float *Wt, float *O,               \
+                                         float *scratch, int NB, int C, int H, int W, int KO,     \
+                                         int R, int S, int st, int pd, int dl)                    \
+    {                                                                                             \
+        const int PH = H + 2 * pd, PW = W + 2 * pd;                                               \
+        const int P = (H + 2 * pd - dl * (R - 1) - 1) / st + 1;                                   \
+        const int Q = (W + 2 * pd - dl * (S - 1) - 1) / st + 1;                                   \
+        pad2d(X, scratch, NB * C, H, W, pd, pd);                                                  \
+        const int nko = (KO + TKO - 1) / TKO;                                                     \
+        _Pragma("omp parallel for schedule(static) collapse(3)")                                  \
+        for (int b = 0; b < NB; ++b)                                                              \
+            for (int kt = 0; kt < nko; ++kt)                                                      \
+                for (int h = 0; h < P; ++h) {                                                     \
+                    const int k0 = kt * TKO;                                                      \
+                    const int nk = (KO - k0) < TKO ? (KO - k0) : TKO;                             \
+                    for (int w0 = 0; w0 < Q; w0 += TW) {                                          \
+                        const int nw = (Q - w0) < TW ? (Q - w0) : TW;                             \
+                        float acc[TKO][TW];                                                       \
+                        memset(acc, 0, sizeof acc);                                               \
+                        for (int rc = 0; rc < C; ++rc)                                            \
+                            for (int rw = 0; rw < S; ++rw)                                        \
+                                for (int rh = 0; rh < R; ++rh) {                                  \
+                                    const float *xr = scratch +                                   \
+                                        (((size_t)b * C + rc) * PH + h * st + rh * dl) * PW +     \
+                                        (size_t)w0 * st + rw * dl;                                \
+                                    for (int kk = 0; kk < nk; ++kk) {                             \
+                                        const float wv =                                          \
+                                            Wt[(((size_t)(k0 + kk) * C + rc) * R + rh) * S + rw]; \
+                                        if (st == 1) {                                            \
+                                            _Pragma("omp simd")                                   \
+                                            for (int ww = 0; ww < TW; ++ww)                       \
+                                                if (ww < nw) acc[kk][ww] += xr[ww] * wv;          \
+                                        } else {                                                  \
+                                            for (int ww = 0; ww < nw; ++ww)                       \
+                                                acc[kk][ww] += xr[(size_t)ww * st] * wv;          \
+                                        }                                                         \
+                                    }                                                             \
+                                }                                                                 \
+                        for (int kk = 0; kk < nk; ++kk)                                           \
+                            for (int ww = 0; ww < nw; ++ww)                                       \
+                                O[(((size_t)b * KO + k0 + kk) * P + h) * Q + w0 + ww] = acc[kk][ww]; \
+                    }                                                                             \
+                }                                                                                 \
+    }
+FTB_DEFINE_CONV(4, 16)
+FTB_DEFINE_CONV(8, 16)
+FTB_DEFINE_CONV(4, 32)
+FTB_DEFINE_CONV(2, 16)
+FTB_DEFINE_CONV(8, 8)
+
+int ftb_conv2d_variants(void) { return 5; }
+void ftb_conv2d_variant_tile(int v, int *tko, int *tw)
+{
+    static const int t[5][2] = {{4, 16}, {8, 16}, {4, 32}, {2, 16}, {8, 8}};
+    *tko = t[v][0];
+    *tw = t[v][1];
+}
+void ftb_conv2d_nchw_v(const float *X, const float *Wt, float *O, float *scratch, int NB, int C,
+                       int H, int W, int KO, int R, int S, int st, int pd, int dl, int v)
+{
+    switch (v) {
+    case 1: conv2d_nchw_8x16(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl); break;
+    case 2: conv2d_nchw_4x32(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl); break;
+    case 3: conv2d_nchw_2x16(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl); break;
+    case 4: conv2d_nchw_8x8(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl); break;
+    default: conv2d_nchw_4x16(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl); break;
+    }
+}
 void ftb_conv2d_nchw(const float *X, const float *Wt, float *O, float *scratch, int NB, int C,
                      int H, int W, int KO, int R, int S, int st, int pd, int dl)
 {
-    const int PH = H + 2 * pd, PW = W + 2 * pd;
-    const int P = (H + 2 * pd - dl * (R - 1) - 1) / st + 1;
-    const int Q = (W + 2 * pd - dl * (S - 1) - 1) / st + 1;
-    pad2d(X, scratch, NB * C, H, W, pd, pd);
-    const int nko = (KO + TKO - 1) / TKO;
-#pragma omp parallel for schedule(static) collapse(3)
-    for (int b = 0; b < NB; ++b)
-        for (int kt = 0; kt < nko; ++kt)
-            for (int h = 0; h < P; ++h) {
-                const int k0 = kt * TKO;
-                const int nk = (KO - k0) < TKO ? (KO - k0) : TKO;
-                for (int w0 = 0; w0 < Q; w0 += TW) {
-                    const int nw = (Q - w0) < TW ? (Q - w0) : TW;
-                    float acc[TKO][TW];
-                    memset(acc, 0, sizeof acc);
-                    for (int rc = 0; rc < C; ++rc)
-                        for (int rw = 0; rw < S; ++rw)
-                            for (int rh = 0; rh < R; ++rh) {
-                                const float *xr = scratch +
-                                    (((size_t)b * C + rc) * PH + h * st + rh * dl) * PW +
-                                    (size_t)w0 * st + rw * dl;
-                                for (int kk = 0; kk < nk; ++kk) {
-                                    const float wv = Wt[(((size_t)(k0 + kk) * C + rc) * R + rh) * S + rw];
-                                    if (st == 1) {
-#pragma omp simd
-                                        for (int ww = 0; ww < TW; ++ww)
-                                            if (ww < nw) acc[kk][ww] += xr[ww] * wv;
-                                    } else {
-                                        for (int ww = 0; ww < nw; ++ww)
-                                            acc[kk][ww] += xr[(size_t)ww * st] * wv;
-                                    }
-                                }
-                            }
-                    for (int kk = 0; kk < nk; ++kk)
-                        for (int ww = 0; ww < nw; ++ww)
-                            O[(((size_t)b * KO + k0 + kk) * P + h) * Q + w0 + ww] = acc[kk][ww];
-                }
-            }
+    conv2d_nchw_4x16(X, Wt, O, scratch, NB, C, H, W, KO, R, S, st, pd, dl);
 }
 
 /* depthwise conv2d NCHW, weight [C][F][R][S] */

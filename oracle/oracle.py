@@ -315,6 +315,42 @@ def baseline_gemm_f32(a, b, out, tk=256):
                                 out.ctypes.data_as(_f32p), a.shape[0], b.shape[1], a.shape[1], tk)
 
 
+def baseline_gemm_f32_tiles():
+    """(rows, columns) of the register tiles the port was built with; the index is the variant."""
+    L = baseline_lib()
+    out = []
+    for v in range(L.ftb_gemm_f32_variants()):
+        ti, tj = ctypes.c_int(), ctypes.c_int()
+        L.ftb_gemm_f32_variant_tile(v, ctypes.byref(ti), ctypes.byref(tj))
+        out.append((ti.value, tj.value))
+    return out
+
+
+def baseline_gemm_f32_v(a, b, out, tk, variant):
+    baseline_lib().ftb_gemm_f32_v(a.ctypes.data_as(_f32p), b.ctypes.data_as(_f32p),
+                                  out.ctypes.data_as(_f32p), a.shape[0], b.shape[1], a.shape[1], tk,
+                                  int(variant))
+
+
+def baseline_conv2d_tiles():
+    """(output channels, output columns) of the convolution's register tiles, by variant index."""
+    L = baseline_lib()
+    out = []
+    for v in range(L.ftb_conv2d_variants()):
+        a, b = ctypes.c_int(), ctypes.c_int()
+        L.ftb_conv2d_variant_tile(v, ctypes.byref(a), ctypes.byref(b))
+        out.append((a.value, b.value))
+    return out
+
+
+def baseline_conv2d_v(x, wt, out, scratch, stride, padding, dilation, variant):
+    nb, c, h, w = x.shape
+    ko, _, r, s = wt.shape
+    baseline_lib().ftb_conv2d_nchw_v(x.ctypes.data_as(_f32p), wt.ctypes.data_as(_f32p),
+                                     out.ctypes.data_as(_f32p), scratch.ctypes.data_as(_f32p),
+                                     nb, c, h, w, ko, r, s, stride, padding, dilation, int(variant))
+
+
 def baseline_gemm_i8(a, b, out, row0=0, row1=None):
     row1 = a.shape[0] if row1 is None else row1
     baseline_lib().ftb_gemm_i8(a.ctypes.data_as(_i8p), b.ctypes.data_as(_i8p),

@@ -890,6 +890,29 @@ def test_builtplan_rejects_mismatched_tensors():
     f.close()
 
 
+def test_schedule_with_the_performance_model_on_device(oracle, tmp_path):
+    """use_model=True end to end on the GPU (flextensor/model.py:448-456, train.py:27-62): a first
+    search measures on the device and leaves its data, the offline trainer fits the ranking
+    network, a second search lets the network rank candidates and measures only its best points;
+    what comes back is a checked, timed kernel that matches the oracle."""
+    from flextensor_amd import train
+    np.random.seed(1)
+    torch.manual_seed(1)
+    key = "gemm_gemm_(512, 256, 512)_rocm(0)"
+    d = str(tmp_path)
+    schedule(key, op_trial=2, graph_trial=1, op_stop=2, parallel=8, number=5, timeout=20, warm_up=(1, 8),
+             verbose=False, method="searching", perf_path=d)
+    assert "performance_judger_data_gemm_op0.txt" in os.listdir(d)
+    train.train_for_schedule(key, perf=True, perf_path=d)
+    assert "performance_judger_model_gemm_op0.pkl" in os.listdir(d)
+    s, bufs, configs = schedule(key, op_trial=3, graph_trial=1, op_stop=3, parallel=8, number=5, timeout=20,
+                                warm_up=(1, 8), verbose=False, method="searching", use_model=True, perf_path=d)
+    a, b = seeded_inputs(bufs, 13)
+    out = run_plan(key, configs, [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+    assert s.specs[-1].kernel == "igemm_f32"
+
+
 @pytest.mark.parametrize("method", ["searching", "q"])
 def test_schedule_on_device_small_gemm(oracle, method):
     """End to end: search a few points on the GPU, replay the winner, check it."""

@@ -174,3 +174,82 @@ def test_schedule_method_q_on_the_four_operator_im2col_graph(tmp_path):
     assert len(configs.op_config_lst) == 4 and configs.op_config_lst[2]["spatial"]
     assert [sp.kernel for sp in s.specs] == ["igemm_f32"]            # folded: fewest kernels wins
     assert configs.graph_config["inline"][0][:2] == [1, 1] and configs.graph_config["merge"][0][3] == 1
+
+
+def _dump_random_batches(path, space, nbatch, per_batch, seed):
+    """A performance-data file as a search leaves it: batches of flattened points with their costs."""
+    rng = np.random.RandomState(seed)
+    wg = WalkerGroup("gemm_op0", space)
+    for _ in range(nbatch):
+        pts, costs = [], []
+        while len(pts) < per_batch:
+            indices = {name: int(rng.randint(sub.size)) for name, sub in space.items()}
+            cfg = wg.to_config(indices)
+            try:
+                cost = _cost(GEMM, Config([cfg], None), 0, 1)
+            except Exception:  # noqa: BLE001  (a point the templates refuse: redrawn, as the warm-up does)
+                if rng.rand() < 0.02:
+                    cost = float("inf")         # a few failed candidates stay in, as in a real dump
+                else:
+                    continue
+            costs.append(cost)
+            pts.append(indices)
+        wg.add_perf_data(pts, costs)
+    wg.dump_performance_data(path)
+    return wg
+
+
+def test_offline_trainer_ranks_a_held_out_dump_better_than_chance(tmp_path):
+    """flextensor/train.py:123-295: a model trained on one dump of measured batches orders the
+    points of another dump of the same task (other random points) clearly better than chance."""
+    from flextensor_amd import train
+    np.random.seed(11)
+    torch.manual_seed(11)
+    space = _space()
+    train_file, held_out = str(tmp_path / "train.txt"), str(tmp_path / "held_out.txt")
+    _dump_random_batches(train_file, space, nbatch=60, per_batch=8, seed=1)
+    _dump_random_batches(held_out, space, nbatch=25, per_batch=8, seed=2)
+    data = train.load_perf_data(train_file)
+    assert len(data) == 60 and train.query_perf_data_info(data) == space.dim
+    flat = train.normalize_perf_data(data)
+    assert len(flat) == 480 and all(c == train.INF_COST or c < 100 for _, c in flat)
+    model_path = str(tmp_path / "perf.pkl")
+    res = train.train_performance_model(train_file, model_path, epoch=12, lr=0.5, override=True)
+    assert os.path.exists(model_path) and res["input_len"] == space.dim
+    with pytest.raises(RuntimeError):
+        train.train_performance_model(train_file, model_path, epoch=1)          # no silent overwrite
+    from flextensor_amd.model import make_performance_model
+    model = make_performance_model(space.dim)
+    model.load_state_dict(torch.load(model_path, weights_only=True))
+    acc = train.pairwise_accuracy(model, train.load_perf_data(held_out))
+    untrained = train.pairwise_accuracy(make_performance_model(space.dim), train.load_perf_data(held_out))
+    assert acc > 0.62 and acc > untrained + 0.05, (acc, untrained)
+    # the reference's active loss (regression of single points) trains as well
+    res = train.train_performance_model(train_file, model_path, epoch=2, lr=0.5, override=True, loss="mse", batch_size=16)
+    assert 0.0 <= res["test_accuracy"] <= 1.0
+
+
+def test_search_dumps_its_measurements_and_train_for_schedule_reads_them(tmp_path):
+    """schedule(perf_path=dir) leaves the measured batches and the walkers' transitions in dir;
+    train_for_schedule (flextensor/train.py:27-62) trains every group from them; a later search
+    with use_model=True picks the trained ranking network up."""
+    from flextensor_amd import train
+    np.random.seed(5)
+    torch.manual_seed(5)
+    d = str(tmp_path)
+    schedule(GEMM, op_trial=6, op_stop=6, graph_trial=2, parallel=4, method="q", evaluator=_cost,
+             warm_up=(2, 8), verbose=False, perf_path=d, warm_start=False)
+    files = os.listdir(d)
+    assert "performance_judger_data_gemm_op0.txt" in files and any(f.startswith("walker_judger_data_") for f in files)
+    batches = train.load_perf_data(os.path.join(d, "performance_judger_data_gemm_op0.txt"))
+    assert sum(len(t) for _, t in batches) >= 16
+    losses = train.train_for_schedule(GEMM, q=True, perf=True, perf_path=d)
+    assert "gemm_op0" in losses and math.isfinite(losses["gemm_op0"])
+    assert "performance_judger_model_gemm_op0.pkl" in os.listdir(d)
+    before = os.path.getmtime(os.path.join(d, "performance_judger_model_gemm_op0.pkl"))
+    s, bufs, configs = schedule(GEMM, op_trial=3, op_stop=3, graph_trial=1, parallel=4, method="searching",
+                                evaluator=_cost, warm_up=(1, 8), verbose=False, use_model=True, perf_path=d)
+    assert os.path.getmtime(os.path.join(d, "performance_judger_model_gemm_op0.pkl")) == before    # loaded, not recreated
+    assert math.isfinite(_cost(GEMM, configs, None, 1))
+    with pytest.raises(ValueError):
+        train.train_for_schedule(GEMM, perf=True)

@@ -1,6 +1,6 @@
 // Direct depthwise conv2d NCHW fp32 kernel template for gfx950, hiprtc-compiled.
 //
-//   O[b][c][h][w] = sum_{r,s} P[b][c / FACT][h*STR + r*DIL][w*STR + s*DIL]
+//   O[b][c][h][w] = sum_{r,s} P[b][c / FACT][h*STRH + r*DILH][w*STRW + s*DILW]
 //                             * Wt[c / FACT][c % FACT][r][s]
 // with P the zero-padded input (padding folded into load predicates), as in
 // flextensor/nn/ops.py:622-678 (weight layout [C][FACT][R][S], ops.py:630).
@@ -23,7 +23,7 @@
 // It needs a same-size 3x3 / stride 1 / dilation 1 / padding 1 layer with
 // FACT == 1 and rows that are multiples of four floats.
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
-// STR, PAD, DIL, FACT, CP x CQ output.
+// STRH/STRW, PADH/PADW, DILH/DILW (rows / columns), FACT, CP x CQ output.
 
 /* Constants arrive as -DFT_<NAME>=value: single-letter macros on the command line
  * would be visible to (and break) the runtime-compilation built-in headers. */
@@ -48,9 +48,12 @@
 #define CW FT_CW
 #define CR FT_CR
 #define CS FT_CS
-#define STR FT_STR
-#define PAD FT_PAD
-#define DIL FT_DIL
+#define STRH FT_STRH
+#define STRW FT_STRW
+#define PADH FT_PADH
+#define PADW FT_PADW
+#define DILH FT_DILH
+#define DILW FT_DILW
 #define FACT FT_FACT
 #define CP FT_CP
 #define CQ FT_CQ
@@ -62,12 +65,12 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #define TILES_H ((CP + TH - 1) / TH)
 #define TILES_W ((CQ + TW - 1) / TW)
 #define ITEMS (PLANES * TILES_H * TILES_W)
-#define IH_T ((TH - 1) * STR + (CR - 1) * DIL + 1)
-#define IW_T ((TW - 1) * STR + (CS - 1) * DIL + 1)
+#define IH_T ((TH - 1) * STRH + (CR - 1) * DILH + 1)
+#define IW_T ((TW - 1) * STRW + (CS - 1) * DILW + 1)
 
 /* 128-bit path: same-size stride-1 convolution whose rows keep 16-byte
  * alignment; the four centre columns of a patch come in as one vector. */
-#if (TW == 4) && (STR == 1) && (CW % 4 == 0) && (CQ == CW) && (PAD + 4 <= IW_T)
+#if (TW == 4) && (STRW == 1) && (CW % 4 == 0) && (CQ == CW) && (PADW + 4 <= IW_T)
 #define VEC_IN 1
 #else
 #define VEC_IN 0
@@ -78,7 +81,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #define VEC_OUT 0
 #endif
 #if SHFL
-#if !(VEC_IN && CS == 3 && DIL == 1 && PAD == 1 && TILES_W <= 64)
+#if !(VEC_IN && CS == 3 && DILW == 1 && PADW == 1 && TILES_W <= 64)
 #error "SHFL needs the 128-bit input path with a 3-wide kernel, dilation 1, padding 1"
 #endif
 #define LPW ((64 / TILES_W) * TILES_W)   /* lanes of a wavefront that carry work */
@@ -87,7 +90,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #endif
 
 #if LDSP > 0
-#if !(STR == 1 && DIL == 1 && CR == 3 && CS == 3 && PAD == 1 && CP == CH && CQ == CW && CW % 4 == 0 && FACT == 1)
+#if !(STRH == 1 && STRW == 1 && DILH == 1 && DILW == 1 && CR == 3 && CS == 3 && PADH == 1 && PADW == 1 && CP == CH && CQ == CW && CW % 4 == 0 && FACT == 1)
 #error "the plane-staged variant needs a same-size 3x3 stride-1 pad-1 layer, FACT 1, CW % 4 == 0"
 #endif
 #define RS (CW + 8)                  /* LDS row: 4 zero floats, CW data, 4 zero floats */
@@ -225,8 +228,8 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 
     const int oh0 = th * TH;
     const int ow0 = tw * TW;
-    const int ih0 = oh0 * STR - PAD;
-    const int iw0 = ow0 * STR - PAD;
+    const int ih0 = oh0 * STRH - PADH;
+    const int iw0 = ow0 * STRW - PADW;
 
     float acc[TH][TW];
 #pragma unroll
@@ -276,7 +279,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     for (int y = 0; y < IH_T; ++y)
 #pragma unroll
         for (int j = 0; j < IW_T; ++j)
-            if (j < PAD || j >= PAD + 4) halo[y][j] = load1(ih0 + y, iw0 + j);
+            if (j < PADW || j >= PADW + 4) halo[y][j] = load1(ih0 + y, iw0 + j);
 #endif
 #endif
 
@@ -300,23 +303,23 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
             const f32x4 v = rows[y];
 #pragma unroll
             for (int j = 0; j < IW_T; ++j)
-                in[j] = (j >= PAD && j < PAD + 4) ? v[(j - PAD) & 3] : halo[y][j];
+                in[j] = (j >= PADW && j < PADW + 4) ? v[(j - PADW) & 3] : halo[y][j];
         }
 #else
 #pragma unroll
         for (int j = 0; j < IW_T; ++j) in[j] = load1(ih0 + y, iw0 + j);
 #endif
-        /* input row y feeds output row i through tap r when y == i*STR + r*DIL */
+        /* input row y feeds output row i through tap r when y == i*STRH + r*DILH */
 #pragma unroll
         for (int i = 0; i < TH; ++i) {
 #pragma unroll
             for (int r = 0; r < CR; ++r) {
-                if (y == i * STR + r * DIL) {
+                if (y == i * STRH + r * DILH) {
 #pragma unroll
                     for (int j = 0; j < TW; ++j)
 #pragma unroll
                         for (int s = 0; s < CS; ++s)
-                            acc[i][j] += in[j * STR + s * DIL] * wreg[r][s];
+                            acc[i][j] += in[j * STRW + s * DILW] * wreg[r][s];
                 }
             }
         }

@@ -4,7 +4,8 @@
 //                   partial sums meet in C with atomics (a kernel rather than
 //                   a memset call so that the launch sequence stays capturable)
 //   copy_f32        streaming copy (bandwidth yardstick, counter calibration)
-//   zero_pad2d_f32  P[b][c][h][w] = X[b][c][h-PAD][w-PAD] inside, 0 outside
+//   zero_pad2d_f32  P[b][c][h][w] = X[b][c][h-PT][w-PL] inside, 0 outside; PT / PB_ rows
+//                   above / below, PL / PR columns left / right
 //                   (flextensor/nn/ops.py:83-117), used when the graph config
 //                   does not inline the padding into the convolution
 //   bias_add_nchw_f32  O[b][c][h][w] = I[b][c][h][w] + bias[c] (ops.py:474-478),
@@ -45,10 +46,14 @@ void copy_f32(const float* __restrict__ src, float* __restrict__ dst, long long 
 #define PB FT_PB
 #define CH FT_CH
 #define CW FT_CW
-#define PAD FT_PAD
-/* shape constants: PB planes (batch*channels), CH x CW input, PAD */
-#define PH (CH + 2 * PAD)
-#define PW (CW + 2 * PAD)
+#define PT FT_PT
+#define PBOT FT_PBOT
+#define PL FT_PL
+#define PR FT_PR
+/* shape constants: PB planes (batch*channels), CH x CW input, padding rows above / below
+ * and columns left / right (flextensor/nn/ops.py:83-117 takes all four) */
+#define PH (CH + PT + PBOT)
+#define PW (CW + PL + PR)
 extern "C" __global__ __launch_bounds__(256)
 void zero_pad2d_f32(const float* __restrict__ X, float* __restrict__ P)
 {
@@ -57,7 +62,7 @@ void zero_pad2d_f32(const float* __restrict__ X, float* __restrict__ P)
     const int w = gid % PW;
     const int h = (gid / PW) % PH;
     const int pl = gid / (PW * PH);
-    const int ih = h - PAD, iw = w - PAD;
+    const int ih = h - PT, iw = w - PL;
     const bool ok = (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
     P[gid] = ok ? X[(size_t)pl * (CH * CW) + ih * CW + iw] : 0.0f;
 }
@@ -75,7 +80,7 @@ void bias_add_nchw_f32(const float* __restrict__ I, const float* __restrict__ bi
 
 #ifdef FT_COLK
 /* convolution geometry: CB batch, CG groups, CC input channels, CH x CW the
- * image as stored (already padded when CPAD is 0 and the padding is its own
+ * image as stored (already padded when CPADH/CPADW are 0 and the padding is its own
  * operator), CR x CS window, CP x CQ output plane, MG output channels per group */
 #define CB FT_CB
 #define CG FT_CG
@@ -84,9 +89,12 @@ void bias_add_nchw_f32(const float* __restrict__ I, const float* __restrict__ bi
 #define CW FT_CW
 #define CR FT_CR
 #define CS FT_CS
-#define CSTR FT_CSTR
-#define CPAD FT_CPAD
-#define CDIL FT_CDIL
+#define CSTRH FT_CSTRH
+#define CSTRW FT_CSTRW
+#define CPADH FT_CPADH
+#define CPADW FT_CPADW
+#define CDILH FT_CDILH
+#define CDILW FT_CDILW
 #define CP FT_CP
 #define CQ FT_CQ
 #define MG FT_MG
@@ -105,8 +113,8 @@ void im2col_nchw_f32(const float* __restrict__ X, float* __restrict__ col)
         const int p = (n % (CP * CQ)) / CQ;
         const int q = n % CQ;
         const int c = g * (CC / CG) + k / (CR * CS);
-        const int ih = p * CSTR + ((k % (CR * CS)) / CS) * CDIL - CPAD;
-        const int iw = q * CSTR + (k % CS) * CDIL - CPAD;
+        const int ih = p * CSTRH + ((k % (CR * CS)) / CS) * CDILH - CPADH;
+        const int iw = q * CSTRW + (k % CS) * CDILW - CPADW;
         const bool ok = (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
         col[gid] = ok ? X[((size_t)b * CC + c) * (CH * CW) + ih * CW + iw] : 0.0f;
     }

@@ -86,6 +86,13 @@ class KernelSpec(object):
 # GEMM view of an operator
 # --------------------------------------------------------------------------
 
+def _conv_steps(attrs):
+    """Stride, padding and dilation constants of a convolution, rows (H) and columns (W)
+    apart: the operator definitions take pairs (flextensor/nn/ops.py:448-459)."""
+    return dict(CSTRH=attrs["stride"][0], CSTRW=attrs["stride"][1], CPADH=attrs["padding"][0],
+                CPADW=attrs["padding"][1], CDILH=attrs["dilation"][0], CDILW=attrs["dilation"][1])
+
+
 class GemmView(object):
     """M, N, K and addressing mode of a contraction-shaped operator."""
 
@@ -115,9 +122,6 @@ class GemmView(object):
             self.dtype = "int8"
         elif kind == "conv2d_nchw":
             a = op.attrs
-            if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
-                    or a["dilation"][0] != a["dilation"][1]:
-                raise NotImplementedError("anisotropic stride/padding/dilation")
             b, kout, p, q = [x.extent for x in op.axis]
             c = op.reduce_axis[0].extent
             s = op.reduce_axis[1].extent  # rw
@@ -129,16 +133,13 @@ class GemmView(object):
             self.mode = 1
             self.dtype = "float32"
             self.groups = groups
-            self.conv = dict(CB=b, CG=groups, CC=c * groups, CH=h, CW=w, CR=r, CS=s, CSTR=a["stride"][0],
-                             CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
+            self.conv = dict(CB=b, CG=groups, CC=c * groups, CH=h, CW=w, CR=r, CS=s, CP=p, CQ=q,
+                             **_conv_steps(a))
         elif kind == "col_gemm":
             # the GEMM stage of an im2col convolution: one [Mg,K] x [K,N] product per group.
             # With the column matrix read through (inlined) it is the implicit GEMM over the
             # image; otherwise a batch of plain GEMMs over the stored columns.
             a = op.attrs
-            if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
-                    or a["dilation"][0] != a["dilation"][1]:
-                raise NotImplementedError("anisotropic stride/padding/dilation")
             groups = op.axis[0].extent
             self.M, self.N = op.axis[1].extent, op.axis[2].extent
             self.K = op.reduce_axis[0].extent
@@ -147,8 +148,7 @@ class GemmView(object):
             b, cin, h, w = a["in_shape"]
             r, sw = a["kernel"]
             p, q = a["out_hw"]
-            self.conv = dict(CB=b, CG=groups, CC=cin, CH=h, CW=w, CR=r, CS=sw, CSTR=a["stride"][0],
-                             CPAD=a["padding"][0], CDIL=a["dilation"][0], CP=p, CQ=q)
+            self.conv = dict(CB=b, CG=groups, CC=cin, CH=h, CW=w, CR=r, CS=sw, CP=p, CQ=q, **_conv_steps(a))
             self.mode = 1 if col_inlined else 0
         else:
             raise InvalidConfig("operator kind %s has no GEMM view" % kind)
@@ -438,8 +438,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     a_bytes = view.groups * view.M * view.K * 4
     if view.mode == 1:
         cv = view.conv
-        grow = 2 * cv["CPAD"] if materialized_pad else 0
-        b_bytes = cv["CB"] * cv["CC"] * (cv["CH"] + grow) * (cv["CW"] + grow) * 4
+        grow_h, grow_w = (2 * cv["CPADH"], 2 * cv["CPADW"]) if materialized_pad else (0, 0)
+        b_bytes = cv["CB"] * cv["CC"] * (cv["CH"] + grow_h) * (cv["CW"] + grow_w) * 4
     else:
         b_bytes = view.groups * view.K * view.N * 4
     if max(a_bytes, b_bytes, view.groups * view.M * view.N * 4) >= 2 ** 31:
@@ -453,9 +453,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     if view.mode == 1:
         conv = dict(view.conv)
         if materialized_pad:
-            conv["CH"] += 2 * conv["CPAD"]
-            conv["CW"] += 2 * conv["CPAD"]
-            conv["CPAD"] = 0
+            conv["CH"] += 2 * conv["CPADH"]
+            conv["CW"] += 2 * conv["CPADW"]
+            conv["CPADH"] = conv["CPADW"] = 0
         D.update(conv)
         if op.kind == "col_gemm" and merged_out is None:
             D.update(COLOUT=1)            # C stays [groups][M][N] for the col2img stage
@@ -509,9 +509,6 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     if waves < 1 or waves * 64 > MAX_THREADS:
         raise InvalidConfig("bad wavefront count")
     a = op.attrs
-    if a["stride"][0] != a["stride"][1] or a["padding"][0] != a["padding"][1] \
-            or a["dilation"][0] != a["dilation"][1]:
-        raise NotImplementedError("anisotropic stride/padding/dilation")
     b, cout, p, q = [x.extent for x in op.axis]
     s_ext = op.reduce_axis[0].extent  # rw
     r_ext = op.reduce_axis[1].extent  # rh
@@ -520,13 +517,13 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         raise InvalidConfig("lane patch larger than the output plane")
     if int(sp[2][0]) != ceil_div(p, th) or int(sp[3][0]) != ceil_div(q, tw):
         raise InvalidConfig("grid level does not match ceil(extent / patch)")
-    pad = a["padding"][0]
+    (st_h, st_w), (pad_h, pad_w), (dl_h, dl_w) = a["stride"], a["padding"], a["dilation"]   # rows, columns
     if materialized_pad:
-        h, w, pad = h + 2 * pad, w + 2 * pad, 0
-    ih_t = (th - 1) * a["stride"][0] + (r_ext - 1) * a["dilation"][0] + 1
-    iw_t = (tw - 1) * a["stride"][0] + (s_ext - 1) * a["dilation"][0] + 1
+        h, w, pad_h, pad_w = h + 2 * pad_h, w + 2 * pad_w, 0, 0
+    ih_t = (th - 1) * st_h + (r_ext - 1) * dl_h + 1
+    iw_t = (tw - 1) * st_w + (s_ext - 1) * dl_w + 1
     # the 128-bit input path requests every row of the patch before the first is used
-    vec_rows = (tw == 4 and a["stride"][0] == 1 and w % 4 == 0 and q == w and pad + 4 <= iw_t)
+    vec_rows = (tw == 4 and st_w == 1 and w % 4 == 0 and q == w and pad_w + 4 <= iw_t)
     if th * tw + (ih_t * iw_t if vec_rows else iw_t) + r_ext * s_ext > 200:
         raise InvalidConfig("lane patch needs too many registers")
     if max(b * c * h * w, b * cout * p * q) * 4 >= 2 ** 31:
@@ -535,32 +532,30 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
     ldsp = int(_special(special, "lds_planes")[0])
     nt_mode = int(_special(special, "nt_store")[0])     # bit 0: non-temporal stores, bit 1: non-temporal loads
+    steps = dict(STRH=st_h, STRW=st_w, PADH=pad_h, PADW=pad_w, DILH=dl_h, DILW=dl_w)
     if ldsp:
         # plane-staged variant: whole planes through LDS in copy order; the lane patch knobs do not apply
-        st, dl = a["stride"][0], a["dilation"][0]
-        if not (st == 1 and dl == 1 and r_ext == 3 and s_ext == 3 and pad == 1 and p == h and q == w
-                and w % 4 == 0 and a["factor"] == 1):
+        if not (st_h == st_w == 1 and dl_h == dl_w == 1 and r_ext == 3 and s_ext == 3 and pad_h == pad_w == 1
+                and p == h and q == w and w % 4 == 0 and a["factor"] == 1):
             raise InvalidConfig("plane staging needs a same-size 3x3 stride-1 pad-1 layer with rows of whole vectors")
         if ldsp < 0 or (ldsp * (h + 2) * (w + 8) + ldsp * 12) * 4 > LDS_BYTES:
             raise InvalidConfig("staged planes do not fit the LDS")
         D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=0, LDSP=ldsp,
-                 CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=1, PAD=1, DIL=1, FACT=1, CP=p, CQ=q)
+                 CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=1, CP=p, CQ=q, **steps)
         return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(b * cout, ldsp), 1, 1),
                            (nt, 1, 1),
                            [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
     shfl = int(_special(special, "halo_shfl")[0])
     tiles_w = ceil_div(q, tw)
     if shfl:
-        vec_in = (tw == 4 and a["stride"][0] == 1 and w % 4 == 0 and q == w and pad + 4 <= iw_t)
-        if not (vec_in and s_ext == 3 and a["dilation"][0] == 1 and pad == 1 and tiles_w <= 64):
-            raise InvalidConfig("the shuffled halo needs the 128-bit input path of a 3x3 pad-1 layer")
+        if not (vec_rows and s_ext == 3 and dl_w == 1 and pad_w == 1 and tiles_w <= 64):
+            raise InvalidConfig("the shuffled halo needs the 128-bit input path of a 3-wide pad-1 layer")
         lanes = (64 // tiles_w) * tiles_w
         grid_x = ceil_div(ceil_div(items, lanes), waves)
     else:
         grid_x = ceil_div(items, nt)
     D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=shfl,
-             CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, STR=a["stride"][0], PAD=pad,
-             DIL=a["dilation"][0], FACT=a["factor"], CP=p, CQ=q)
+             CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=a["factor"], CP=p, CQ=q, **steps)
     return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
                        (nt, 1, 1),
                        [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
@@ -568,11 +563,9 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
 
 def _lower_pad(op, out_name, in_names):
     b, c, ph, pw = [x.extent for x in op.axis]
-    pt, pb, pl, pr = op.attrs["padding"]
-    if not (pt == pb == pl == pr):
-        raise NotImplementedError("asymmetric padding")
-    h, w = ph - 2 * pt, pw - 2 * pt
-    D = dict(PADK=1, PB=b * c, CH=h, CW=w, PAD=pt)
+    pt, pb, pl, pr = op.attrs["padding"]          # rows above / below, columns left / right
+    h, w = ph - pt - pb, pw - pl - pr
+    D = dict(PADK=1, PB=b * c, CH=h, CW=w, PT=pt, PBOT=pb, PL=pl, PR=pr)
     n = b * c * ph * pw
     return [KernelSpec("elementwise.hip", "zero_pad2d_f32", D, (ceil_div(n, 256), 1, 1),
                        (256, 1, 1), [("buf", in_names[0]), ("buf", out_name)])]
@@ -593,17 +586,14 @@ def _lower_bias(op, out_name, in_names):
 
 
 def _conv_defines(attrs, materialized_pad):
-    if attrs["stride"][0] != attrs["stride"][1] or attrs["padding"][0] != attrs["padding"][1] \
-            or attrs["dilation"][0] != attrs["dilation"][1]:
-        raise NotImplementedError("anisotropic stride/padding/dilation")
     b, cin, h, w = attrs["in_shape"]
-    pad = attrs["padding"][0]
+    steps = _conv_steps(attrs)
     if materialized_pad:
-        h, w, pad = h + 2 * pad, w + 2 * pad, 0
+        h, w = h + 2 * steps["CPADH"], w + 2 * steps["CPADW"]
+        steps["CPADH"] = steps["CPADW"] = 0
     groups = attrs["groups"]
     return dict(COLK=1, CB=b, CG=groups, CC=cin, CH=h, CW=w, CR=attrs["kernel"][0], CS=attrs["kernel"][1],
-                CSTR=attrs["stride"][0], CPAD=pad, CDIL=attrs["dilation"][0], CP=attrs["out_hw"][0],
-                CQ=attrs["out_hw"][1], MG=attrs["out_channel"] // groups)
+                CP=attrs["out_hw"][0], CQ=attrs["out_hw"][1], MG=attrs["out_channel"] // groups, **steps)
 
 
 def _lower_im2col(op, out_name, in_names, materialized_pad):
@@ -618,7 +608,8 @@ def _lower_col2img(op, out_name, in_names):
     b, c, p, q = [x.extent for x in op.axis]
     g, mg, _ = op.input_tensors[0].shape
     # only the output geometry matters to this kernel; the image constants are placeholders
-    D = dict(COLK=1, CB=b, CG=g, CC=g, CH=1, CW=1, CR=1, CS=1, CSTR=1, CPAD=0, CDIL=1, CP=p, CQ=q, MG=mg)
+    D = dict(COLK=1, CB=b, CG=g, CC=g, CH=1, CW=1, CR=1, CS=1, CSTRH=1, CSTRW=1, CPADH=0, CPADW=0,
+             CDILH=1, CDILW=1, CP=p, CQ=q, MG=mg)
     total = b * c * p * q
     return [KernelSpec("elementwise.hip", "col2img_nchw_f32", D,
                        (min(ceil_div(total, 256), 16384), 1, 1), (256, 1, 1),

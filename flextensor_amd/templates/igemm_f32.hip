@@ -324,13 +324,17 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #define CW FT_CW
 #define CR FT_CR
 #define CS FT_CS
-#define CSTR FT_CSTR
-#define CPAD FT_CPAD
-#define CDIL FT_CDIL
+#define CSTRH FT_CSTRH
+#define CSTRW FT_CSTRW
+#define CPADH FT_CPADH
+#define CPADW FT_CPADW
+#define CDILH FT_CDILH
+#define CDILW FT_CDILW
 #define CP FT_CP
 #define CQ FT_CQ
 /* conv geometry, all compile-time: input [CB][CC][CH][CW], kernel CR x CS,
- * stride CSTR, padding CPAD, dilation CDIL, output CP x CQ. */
+ * stride CSTRH x CSTRW, padding CPADH x CPADW, dilation CDILH x CDILW (rows x
+ * columns, flextensor/nn/ops.py:448-459 takes pairs), output CP x CQ. */
 #define OHW (CP * CQ)
 #define A_BYTES (CG * M * K * 4)
 #define B_BYTES (CB * CC * CH * CW * 4)
@@ -589,8 +593,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         const int nn = px_ok[e] ? n : 0;
         const int b = nn / OHW;
         const int p = nn % OHW;
-        px_h[e] = (p / CQ) * CSTR - CPAD;
-        px_w[e] = (p % CQ) * CSTR - CPAD;
+        px_h[e] = (p / CQ) * CSTRH - CPADH;
+        px_w[e] = (p % CQ) * CSTRW - CPADW;
         px_off[e] = b * (CC * CH * CW) + gi * ((CC / CG) * CH * CW);
     }
 #endif
@@ -635,8 +639,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #elif KHOIST
         const int cl = b_row[e] / (CR * CS);
         const int rs = b_row[e] % (CR * CS);
-        const int ih = px_h[e] + (rs / CS) * CDIL;
-        const int iw = px_w[e] + (rs % CS) * CDIL;
+        const int ih = px_h[e] + (rs / CS) * CDILH;
+        const int iw = px_w[e] + (rs % CS) * CDILW;
         ok = ok && px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
         b_voff[e] = ok ? (unsigned)(px_off[e] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
 #else
@@ -678,8 +682,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int k = k0 + b_row[e];
             const int c = k / (CR * CS);
             const int rs = k % (CR * CS);
-            const int ih = px_h[e] + (rs / CS) * CDIL;
-            const int iw = px_w[e] + (rs % CS) * CDIL;
+            const int ih = px_h[e] + (rs / CS) * CDILH;
+            const int iw = px_w[e] + (rs % CS) * CDILW;
             bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
             if (KP != K) ok = ok && (k < K);
             const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
@@ -848,8 +852,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int k = k0 + b_row[e];
             const int c = k / (CR * CS);
             const int rs = k % (CR * CS);
-            const int ih = px_h[e] + (rs / CS) * CDIL;
-            const int iw = px_w[e] + (rs % CS) * CDIL;
+            const int ih = px_h[e] + (rs / CS) * CDILH;
+            const int iw = px_w[e] + (rs % CS) * CDILW;
             bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
             if (KP != K) ok = ok && (k < K);
             const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;

@@ -85,17 +85,23 @@ def zero_pad2d_c(x, padding):
     return out
 
 
+def _hw(v):
+    """int or (rows, columns) pair, as flextensor/nn/ops.py:448-456 accepts."""
+    return (int(v), int(v)) if isinstance(v, (int, np.integer)) else (int(v[0]), int(v[1]))
+
+
 def conv2d_nchw_c(x, wt, stride=1, padding=0, dilation=1, groups=1, fma=True):
     x, xp = _f32(x)
     wt, wp = _f32(wt)
     nb, c, h, w = x.shape
     ko, cg, r, s = wt.shape
     assert cg * groups == c
-    p = conv_out_size(h, padding, dilation, r, stride)
-    q = conv_out_size(w, padding, dilation, s, stride)
+    (sh, sw), (ph, pw), (dh, dw) = _hw(stride), _hw(padding), _hw(dilation)
+    p = conv_out_size(h, ph, dh, r, sh)
+    q = conv_out_size(w, pw, dw, s, sw)
     out = np.empty((nb, ko, p, q), dtype=np.float32)
-    rc = lib().ft_conv2d_nchw(xp, wp, out.ctypes.data_as(_f32p), nb, c, h, w, ko, r, s, stride,
-                              stride, padding, padding, dilation, dilation, groups, int(fma))
+    rc = lib().ft_conv2d_nchw(xp, wp, out.ctypes.data_as(_f32p), nb, c, h, w, ko, r, s, sh,
+                              sw, ph, pw, dh, dw, groups, int(fma))
     if rc != 0:
         raise MemoryError("oracle conv2d scratch")
     return out
@@ -107,11 +113,12 @@ def depthwise_nchw_c(x, wt, stride=1, padding=0, dilation=1, fma=True):
     nb, c, h, w = x.shape
     c2, f, r, s = wt.shape
     assert c2 == c
-    p = conv_out_size(h, padding, dilation, r, stride)
-    q = conv_out_size(w, padding, dilation, s, stride)
+    (sh, sw), (ph, pw), (dh, dw) = _hw(stride), _hw(padding), _hw(dilation)
+    p = conv_out_size(h, ph, dh, r, sh)
+    q = conv_out_size(w, pw, dw, s, sw)
     out = np.empty((nb, c * f, p, q), dtype=np.float32)
-    rc = lib().ft_depthwise_nchw(xp, wp, out.ctypes.data_as(_f32p), nb, c, h, w, f, r, s, stride,
-                                 stride, padding, padding, dilation, dilation, int(fma))
+    rc = lib().ft_depthwise_nchw(xp, wp, out.ctypes.data_as(_f32p), nb, c, h, w, f, r, s, sh,
+                                 sw, ph, pw, dh, dw, int(fma))
     if rc != 0:
         raise MemoryError("oracle depthwise scratch")
     return out

@@ -66,7 +66,7 @@ def test_default_lowering_of_baseline_tasks():
             assert all(g >= 1 for g in spec.grid)
     s, _ = schedule_with_config(CONV, Config([], None))
     d = s.specs[-1].defines
-    assert d["MODE"] == 1 and (d["M"], d["N"], d["K"]) == (64, 3136, 576) and d["CPAD"] == 1
+    assert d["MODE"] == 1 and (d["M"], d["N"], d["K"]) == (64, 3136, 576) and d["CPADH"] == 1 and d["CPADW"] == 1
     assert [a[1] for a in s.specs[-1].args] == ["in1", "in0", "out"]  # A = weight, B = image
     assert s.intermediates == {}
 
@@ -79,7 +79,7 @@ def test_graph_config_not_inlined_materialises_padding():
     assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "igemm_f32"]
     assert s.intermediates == {"tmp0": ((1, 64, 58, 58), "float32")}
     d = s.specs[-1].defines
-    assert d["CPAD"] == 0 and d["CH"] == 58 and d["CW"] == 58
+    assert d["CPADH"] == 0 and d["CPADW"] == 0 and d["CH"] == 58 and d["CW"] == 58
     assert [a[1] for a in s.specs[-1].args] == ["in1", "tmp0", "out"]
     g["inline"] = [[1, 1]]
     with pytest.raises(ValueError):
@@ -225,13 +225,13 @@ def test_gemm_conv2d_graph_flags_choose_the_kernel_sequence():
     assert s.specs[0].defines["COLOUT"] == 1 and s.intermediates == {"tmp2": ((1, 512, 3136), "float32")}
     s = plan([0, 0, 0, 0], [0, 0, 0, 0])
     assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "im2col_nchw_f32", "igemm_f32", "col2img_nchw_f32"]
-    assert s.specs[1].defines["CH"] == 58 and s.specs[1].defines["CPAD"] == 0      # reads the padded image
+    assert s.specs[1].defines["CH"] == 58 and s.specs[1].defines["CPADH"] == 0      # reads the padded image
     assert s.specs[2].defines["MODE"] == 0 and [a[1] for a in s.specs[2].args] == ["in1", "tmp1", "tmp2"]
     s = plan([1, 0, 0, 0], [0, 0, 0, 0])
-    assert s.specs[0].kernel == "im2col_nchw_f32" and s.specs[0].defines["CH"] == 56 and s.specs[0].defines["CPAD"] == 1
+    assert s.specs[0].kernel == "im2col_nchw_f32" and s.specs[0].defines["CH"] == 56 and s.specs[0].defines["CPADH"] == 1
     s = plan([0, 1, 0, 0], [0, 0, 0, 1])
     assert [x.kernel for x in s.specs] == ["zero_pad2d_f32", "igemm_f32"]
-    assert s.specs[1].defines["CPAD"] == 0 and s.specs[1].defines["CH"] == 58 and "COLOUT" not in s.specs[1].defines
+    assert s.specs[1].defines["CPADH"] == 0 and s.specs[1].defines["CH"] == 58 and "COLOUT" not in s.specs[1].defines
     # one image: [groups][M][P*Q] is NCHW already, so the GEMM over stored columns writes the output itself
     s = plan([1, 0, 0, 0], [0, 0, 0, 1])
     assert [x.kernel for x in s.specs] == ["im2col_nchw_f32", "igemm_f32"] and s.specs[1].args[2] == ("buf", "out")

@@ -87,6 +87,32 @@ def test_conv2d_vs_torch(oracle):
         assert rel(oracle.conv2d_nchw_np(x, wt, st, p, d, g), ref) < 1e-12
 
 
+def test_conv2d_and_depthwise_with_row_column_pairs_vs_torch(oracle):
+    """stride, padding and dilation given as (rows, columns) pairs (flextensor/nn/ops.py:448-459):
+    each of the three differs between the axes, so a swapped or shared pair changes the output
+    size or the values."""
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    rng = np.random.default_rng(8)
+    for (n, c, h, w, k, r, s_, st, p, d, g) in [
+            (2, 6, 11, 14, 8, 3, 3, (2, 1), (1, 2), (1, 2), 1),
+            (1, 4, 13, 9, 6, 3, 5, (1, 2), (0, 2), (2, 1), 2),
+            (3, 5, 8, 8, 5, 1, 3, (1, 1), (0, 1), (1, 1), 1)]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (k, c // g, r, s_)).astype(np.float32)
+        ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(), None, st, p, d, g).numpy()
+        out = oracle.conv2d_nchw_c(x, wt, st, p, d, g)
+        assert out.shape == ref.shape and rel(out, ref) < 1e-6
+    for (n, c, h, w, f, r, s_, st, p, d) in [(2, 6, 11, 14, 2, 3, 3, (2, 1), (1, 2), (1, 2)),
+                                             (1, 5, 9, 12, 1, 3, 3, (1, 2), (1, 0), (1, 1))]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (c, f, r, s_)).astype(np.float32)
+        ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt.reshape(c * f, 1, r, s_)).double(),
+                       None, st, p, d, c).numpy()
+        out = oracle.depthwise_nchw_c(x, wt, st, p, d)
+        assert out.shape == ref.shape and rel(out, ref) < 1e-6
+
+
 def test_conv2d_bias_vs_torch(oracle):
     """conv + per-channel bias, as the reference's own test runs it
     (flextensor/test/test_ops.py:85-115 passes a bias to both sides)."""

@@ -125,7 +125,7 @@ def run_default_schedule(ops, tensors, stream=0):
         K = op.reduce_axis[0].extent
         for b in range(nb):
             args = [rt.ptr(tensors[0][b]), rt.ptr(tensors[1][b]), rt.ptr(out[b]), i32(M), i32(N), i32(K),
-                    i32(1 if op.attrs.get("transposeB") else 0), i32(0)]
+                    i32(1 if op.attrs.get("transposeB") else 0), i32(1 if op.attrs.get("transposeA") else 0)]
             _naive("gemm_f32_naive").launch(_grid1d(M * N), (256, 1, 1), args, stream=stream)
         return
     if op.kind == "gemm":

@@ -200,15 +200,16 @@ def gemm(A, B, transposeA=False, transposeB=False):
 
 
 def batch_gemm(A, B, transposeA=False, transposeB=False):
-    """C[b,i,j] = sum_k A[b,i,k] * B[b,k,j] (B optionally stored [b,j,k]).
+    """C[b,i,j] = sum_k A[b,i,k] * B[b,k,j] (A optionally stored [b,k,i], B [b,j,k]).
 
     Follows flextensor/nn/ops.py:1111-1158.
     """
-    if transposeA:
-        raise NotImplementedError("transposeA is not on the tuned path")
     if A.shape[0] != B.shape[0]:
         raise ValueError("batch extents differ: %d vs %d" % (A.shape[0], B.shape[0]))
-    batch, m, k_a = A.shape
+    if transposeA:
+        batch, k_a, m = A.shape
+    else:
+        batch, m, k_a = A.shape
     if transposeB:
         _, n, k_b = B.shape
     else:
@@ -218,7 +219,7 @@ def batch_gemm(A, B, transposeA=False, transposeB=False):
     axis = [IterVar("b", batch), IterVar("i", m), IterVar("j", n)]
     raxis = [IterVar("k", k_a, "reduce")]
     op = ComputeOp("compute", "batch_gemm", (batch, m, n), A.dtype, axis, raxis, [A, B],
-                   {"transposeA": False, "transposeB": bool(transposeB)})
+                   {"transposeA": bool(transposeA), "transposeB": bool(transposeB)})
     return op.output(0)
 
 

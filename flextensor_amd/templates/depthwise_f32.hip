@@ -37,6 +37,11 @@
 #else
 #define NT_LOAD 0
 #endif
+#ifdef FT_IPL
+#define IPL FT_IPL        /* patches per lane */
+#else
+#define IPL 1
+#endif
 #ifdef FT_LDSP
 #define LDSP FT_LDSP
 #else
@@ -185,148 +190,168 @@ extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                    float* __restrict__ O)
 {
-#if SHFL
-    const int lane = threadIdx.x & 63;
-    const int gid = ((blockIdx.x * NT + threadIdx.x) >> 6) * LPW + lane;
-    /* idle lanes stay alive (DPP reads their registers) but load and store nothing */
-    const bool live = (lane < LPW) && (gid < ITEMS);
-#else
-    const int gid = blockIdx.x * NT + threadIdx.x;
-    const bool live = gid < ITEMS;
-#endif
-    const int tw = gid % TILES_W;
-    const int th = (gid / TILES_W) % TILES_H;
-    const int plane = gid / (TILES_W * TILES_H);
-    const int b = plane / (CC * FACT);
-    const int co = plane % (CC * FACT);
-    const int ci = co / FACT;
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(Wt), 0, W_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, O_BYTES, 0x00020000);
-    const int xplane = (b * CC + ci) * (CH * CW);      /* first element of the input plane */
-    const int oplane = plane * (CP * CQ);
 
-    float wreg[CR][CS];
-    {
-        /* the kernel's CR*CS taps: 128-bit loads (dword-aligned is enough for buffer loads) and a tail */
-        const unsigned wo = live ? (unsigned)(co * (CR * CS)) * 4u : OOB;
-        float wflat[(CR * CS + 3) / 4 * 4];
-#pragma unroll
-        for (int t = 0; t + 4 <= CR * CS; t += 4) {
-            const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, (int)wo, t * 4, 0));
-            wflat[t] = v[0]; wflat[t + 1] = v[1]; wflat[t + 2] = v[2]; wflat[t + 3] = v[3];
-        }
-#pragma unroll
-        for (int t = (CR * CS) / 4 * 4; t < CR * CS; ++t)
-            wflat[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rw, (int)wo, t * 4, 0));
-#pragma unroll
-        for (int r = 0; r < CR; ++r)
-#pragma unroll
-            for (int s = 0; s < CS; ++s)
-                wreg[r][s] = wflat[r * CS + s];
-    }
-
-    const int oh0 = th * TH;
-    const int ow0 = tw * TW;
-    const int ih0 = oh0 * STRH - PADH;
-    const int iw0 = ow0 * STRW - PADW;
-
-    float acc[TH][TW];
-#pragma unroll
-    for (int i = 0; i < TH; ++i)
-#pragma unroll
-        for (int j = 0; j < TW; ++j)
-            acc[i][j] = 0.0f;
-
-    auto store_row = [&](int i) {
-        const int oh = oh0 + i;
-        const bool row_ok = live && (CP % TH == 0 || oh < CP);
-#if VEC_OUT
-        f32x4 v;
-        v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
-        const unsigned vo = row_ok ? (unsigned)(oplane + oh * CQ + ow0) * 4u : OOB;
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ro, (int)vo, 0, ST_AUX);
-#else
-#pragma unroll
-        for (int j = 0; j < TW; ++j) {
-            const bool ok = row_ok && (CQ % TW == 0 || ow0 + j < CQ);
-            const unsigned vo = ok ? (unsigned)(oplane + oh * CQ + ow0 + j) * 4u : OOB;
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc[i][j]), ro, (int)vo, 0, ST_AUX);
-        }
-#endif
-    };
-    /* one element of input row ih (any int), column iw (any int); zero outside the image */
-    auto load1 = [&](int ih, int iw) -> float {
-        const bool ok = live && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-        const unsigned vo = ok ? (unsigned)(xplane + ih * CW + iw) * 4u : OOB;
-        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)vo, 0, LD_AUX));
-    };
+    /* A lane works on IPL patches, NT lanes (LPW per wavefront) apart, so that a
+     * workgroup covers one contiguous run of IPL * (lanes that carry work)
+     * patches. Everything a patch needs is requested first, for all IPL
+     * patches (phase 1); the arithmetic and the stores follow (phase 2): a
+     * lane keeps IPL * (IH_T + taps) loads in flight, and fewer, longer-lived
+     * wavefronts move the same bytes. */
+    bool live[IPL];
+    int tw[IPL], ovo[IPL], oh0[IPL];
+    float wreg[IPL][CR][CS];
 #if (SHFL || VEC_IN)
-    /* the four centre columns of input row ih0 + y */
-    auto load_row4 = [&](int y) -> f32x4 {
-        const int ih = ih0 + y;
-        const bool row_ok = live && (unsigned)ih < (unsigned)CH;
-        const unsigned vo = row_ok ? (unsigned)(xplane + ih * CW + ow0) * 4u : OOB;
-        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo, 0, LD_AUX));
-    };
-    f32x4 rows[IH_T];
-#pragma unroll
-    for (int y = 0; y < IH_T; ++y) rows[y] = load_row4(y);
+    f32x4 rows[IPL][IH_T];
 #if !SHFL
-    /* the halo columns left and right of the centre vector */
-    float halo[IH_T][IW_T];
-#pragma unroll
-    for (int y = 0; y < IH_T; ++y)
-#pragma unroll
-        for (int j = 0; j < IW_T; ++j)
-            if (j < PADW || j >= PADW + 4) halo[y][j] = load1(ih0 + y, iw0 + j);
+    float halo[IPL][IH_T][IW_T];
 #endif
+#else
+    float in_all[IPL][IH_T][IW_T];
 #endif
 
 #pragma unroll
-    for (int y = 0; y < IH_T; ++y) {
-        float in[IW_T];
+    for (int k = 0; k < IPL; ++k) {
 #if SHFL
+        const int lane = threadIdx.x & 63;
+        const int gid = (((blockIdx.x * IPL + k) * NT + threadIdx.x) >> 6) * LPW + lane;
+        /* idle lanes stay alive (DPP reads their registers) but load and store nothing */
+        live[k] = (lane < LPW) && (gid < ITEMS);
+#else
+        const int gid = (blockIdx.x * IPL + k) * NT + threadIdx.x;
+        live[k] = gid < ITEMS;
+#endif
+        tw[k] = gid % TILES_W;
+        const int th = (gid / TILES_W) % TILES_H;
+        const int plane = gid / (TILES_W * TILES_H);
+        const int b = plane / (CC * FACT);
+        const int co = plane % (CC * FACT);
+        const int ci = co / FACT;
+        const int xplane = (b * CC + ci) * (CH * CW);      /* first element of the input plane */
+        oh0[k] = th * TH;
+        const int ow0 = tw[k] * TW;
+        const int ih0 = oh0[k] * STRH - PADH;
+        const int iw0 = ow0 * STRW - PADW;
+        ovo[k] = plane * (CP * CQ) + oh0[k] * CQ + ow0;     /* first output element of the patch */
         {
-            const f32x4 v = rows[y];
-            /* column ow0-1 is the last column of the lane below, column ow0+4
-             * the first column of the lane above; image borders read zero */
-            const float v0 = v[0], v3 = v[3];
-            const int lft = __builtin_amdgcn_update_dpp(0, __float_as_int(v3), 0x138, 0xf, 0xf, false);
-            const int rgt = __builtin_amdgcn_update_dpp(0, __float_as_int(v0), 0x130, 0xf, 0xf, false);
-            in[0] = (tw > 0) ? __int_as_float(lft) : 0.0f;
-            in[1] = v[0]; in[2] = v[1]; in[3] = v[2]; in[4] = v[3];
-            in[5] = (tw < TILES_W - 1) ? __int_as_float(rgt) : 0.0f;
+            /* the kernel's CR*CS taps: 128-bit loads (dword-aligned is enough for buffer loads) and a tail */
+            const unsigned wo = live[k] ? (unsigned)(co * (CR * CS)) * 4u : OOB;
+            float wflat[(CR * CS + 3) / 4 * 4];
+#pragma unroll
+            for (int t = 0; t + 4 <= CR * CS; t += 4) {
+                const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, (int)wo, t * 4, 0));
+                wflat[t] = v[0]; wflat[t + 1] = v[1]; wflat[t + 2] = v[2]; wflat[t + 3] = v[3];
+            }
+#pragma unroll
+            for (int t = (CR * CS) / 4 * 4; t < CR * CS; ++t)
+                wflat[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rw, (int)wo, t * 4, 0));
+#pragma unroll
+            for (int r = 0; r < CR; ++r)
+#pragma unroll
+                for (int s = 0; s < CS; ++s)
+                    wreg[k][r][s] = wflat[r * CS + s];
         }
-#elif VEC_IN
-        {
-            const f32x4 v = rows[y];
+        /* one element of input row ih (any int), column iw (any int); zero outside the image */
+        auto load1 = [&](int ih, int iw) -> float {
+            const bool ok = live[k] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+            const unsigned vo = ok ? (unsigned)(xplane + ih * CW + iw) * 4u : OOB;
+            return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rx, (int)vo, 0, LD_AUX));
+        };
+#if (SHFL || VEC_IN)
+#pragma unroll
+        for (int y = 0; y < IH_T; ++y) {
+            /* the four centre columns of input row ih0 + y */
+            const int ih = ih0 + y;
+            const bool row_ok = live[k] && (unsigned)ih < (unsigned)CH;
+            const unsigned vo = row_ok ? (unsigned)(xplane + ih * CW + ow0) * 4u : OOB;
+            rows[k][y] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo, 0, LD_AUX));
+        }
+#if !SHFL
+        /* the halo columns left and right of the centre vector */
+#pragma unroll
+        for (int y = 0; y < IH_T; ++y)
 #pragma unroll
             for (int j = 0; j < IW_T; ++j)
-                in[j] = (j >= PADW && j < PADW + 4) ? v[(j - PADW) & 3] : halo[y][j];
-        }
+                if (j < PADW || j >= PADW + 4) halo[k][y][j] = load1(ih0 + y, iw0 + j);
+#endif
 #else
 #pragma unroll
-        for (int j = 0; j < IW_T; ++j) in[j] = load1(ih0 + y, iw0 + j);
+        for (int y = 0; y < IH_T; ++y)
+#pragma unroll
+            for (int j = 0; j < IW_T; ++j) in_all[k][y][j] = load1(ih0 + y, iw0 + j);
 #endif
-        /* input row y feeds output row i through tap r when y == i*STRH + r*DILH */
+    }
+
 #pragma unroll
-        for (int i = 0; i < TH; ++i) {
+    for (int k = 0; k < IPL; ++k) {
+        float acc[TH][TW];
 #pragma unroll
-            for (int r = 0; r < CR; ++r) {
-                if (y == i * STRH + r * DILH) {
+        for (int i = 0; i < TH; ++i)
 #pragma unroll
-                    for (int j = 0; j < TW; ++j)
+            for (int j = 0; j < TW; ++j)
+                acc[i][j] = 0.0f;
 #pragma unroll
-                        for (int s = 0; s < CS; ++s)
-                            acc[i][j] += in[j * STRW + s * DILW] * wreg[r][s];
+        for (int y = 0; y < IH_T; ++y) {
+            float in[IW_T];
+#if SHFL
+            {
+                const f32x4 v = rows[k][y];
+                /* column ow0-1 is the last column of the lane below, column ow0+4
+                 * the first column of the lane above; image borders read zero */
+                const float v0 = v[0], v3 = v[3];
+                const int lft = __builtin_amdgcn_update_dpp(0, __float_as_int(v3), 0x138, 0xf, 0xf, false);
+                const int rgt = __builtin_amdgcn_update_dpp(0, __float_as_int(v0), 0x130, 0xf, 0xf, false);
+                in[0] = (tw[k] > 0) ? __int_as_float(lft) : 0.0f;
+                in[1] = v[0]; in[2] = v[1]; in[3] = v[2]; in[4] = v[3];
+                in[5] = (tw[k] < TILES_W - 1) ? __int_as_float(rgt) : 0.0f;
+            }
+#elif VEC_IN
+            {
+                const f32x4 v = rows[k][y];
+#pragma unroll
+                for (int j = 0; j < IW_T; ++j)
+                    in[j] = (j >= PADW && j < PADW + 4) ? v[(j - PADW) & 3] : halo[k][y][j];
+            }
+#else
+#pragma unroll
+            for (int j = 0; j < IW_T; ++j) in[j] = in_all[k][y][j];
+#endif
+            /* input row y feeds output row i through tap r when y == i*STRH + r*DILH */
+#pragma unroll
+            for (int i = 0; i < TH; ++i) {
+#pragma unroll
+                for (int r = 0; r < CR; ++r) {
+                    if (y == i * STRH + r * DILH) {
+#pragma unroll
+                        for (int j = 0; j < TW; ++j)
+#pragma unroll
+                            for (int s = 0; s < CS; ++s)
+                                acc[i][j] += in[j * STRW + s * DILW] * wreg[k][r][s];
+                    }
                 }
             }
         }
-    }
-    /* stores last: vector memory operations retire in issue order, so a load
-     * issued behind a store would have to wait for the store's round trip */
+        /* stores behind every load of the kernel: vector memory operations retire in issue
+         * order, so a load issued behind a store would have to wait for the store's round trip */
 #pragma unroll
-    for (int i = 0; i < TH; ++i) store_row(i);
+        for (int i = 0; i < TH; ++i) {
+            const bool row_ok = live[k] && (CP % TH == 0 || oh0[k] + i < CP);
+#if VEC_OUT
+            f32x4 v;
+            v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
+            const unsigned vo = row_ok ? (unsigned)(ovo[k] + i * CQ) * 4u : OOB;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ro, (int)vo, 0, ST_AUX);
+#else
+#pragma unroll
+            for (int j = 0; j < TW; ++j) {
+                const bool ok = row_ok && (CQ % TW == 0 || tw[k] * TW + j < CQ);
+                const unsigned vo = ok ? (unsigned)(ovo[k] + i * CQ + j) * 4u : OOB;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc[i][j]), ro, (int)vo, 0, ST_AUX);
+            }
+#endif
+        }
+    }
 }
 #endif

@@ -111,6 +111,7 @@ class GemmView(object):
         elif kind == "batch_gemm":
             # one GEMM per batch entry: the batch index is the group index of the kernel
             self.groups = op.axis[0].extent
+            self.trans_a = bool(op.attrs.get("transposeA"))
             self.M, self.N = op.axis[1].extent, op.axis[2].extent
             self.K = op.reduce_axis[0].extent
             self.mode = 2 if op.attrs.get("transposeB") else 0
@@ -239,6 +240,7 @@ SPECIAL_DEFAULTS = {
     "nt_store": [0],
     "halo_shfl": [0],
     "lds_planes": [0],
+    "lane_items": [1],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -260,7 +262,8 @@ def special_knobs(kind):
     if kind == "gemm_int8":
         return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
-        return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]]}
+        return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]],
+                "lane_items": [[1], [2], [3], [4], [6], [8]]}
     return {}
 
 
@@ -524,8 +527,12 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     iw_t = (tw - 1) * st_w + (s_ext - 1) * dl_w + 1
     # the 128-bit input path requests every row of the patch before the first is used
     vec_rows = (tw == 4 and st_w == 1 and w % 4 == 0 and q == w and pad_w + 4 <= iw_t)
-    if th * tw + (ih_t * iw_t if vec_rows else iw_t) + r_ext * s_ext > 200:
-        raise InvalidConfig("lane patch needs too many registers")
+    # lane_items: patches per lane, all requested before the first is computed
+    ipl = int(_special(special, "lane_items")[0])
+    if ipl < 1 or ipl > 16:
+        raise InvalidConfig("lane_items is 1 .. 16")
+    if th * tw + ipl * ((ih_t * iw_t if vec_rows else ih_t * iw_t) + r_ext * s_ext) > 220:
+        raise InvalidConfig("lane patches need too many registers")
     if max(b * c * h * w, b * cout * p * q) * 4 >= 2 ** 31:
         raise InvalidConfig("tensors of 2 GiB or more are not addressable by the buffer accesses")
     nt = waves * 64
@@ -551,11 +558,13 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         if not (vec_rows and s_ext == 3 and dl_w == 1 and pad_w == 1 and tiles_w <= 64):
             raise InvalidConfig("the shuffled halo needs the 128-bit input path of a 3-wide pad-1 layer")
         lanes = (64 // tiles_w) * tiles_w
-        grid_x = ceil_div(ceil_div(items, lanes), waves)
+        grid_x = ceil_div(ceil_div(items, lanes), waves * ipl)
     else:
-        grid_x = ceil_div(items, nt)
+        grid_x = ceil_div(items, nt * ipl)
     D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=shfl,
              CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=a["factor"], CP=p, CQ=q, **steps)
+    if ipl > 1:
+        D.update(IPL=ipl)
     return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
                        (nt, 1, 1),
                        [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]

@@ -511,6 +511,35 @@ def test_batch_gemm_vs_oracle(oracle, args, kn, pad):
     assert rel(out.cpu().numpy(), ref) <= TOL
 
 
+def test_batch_gemm_transposed_operands_vs_oracle(oracle):
+    """batch_gemm with A stored [b,k,i] and / or B stored [b,j,k] (flextensor/nn/ops.py:1131-1145)."""
+    from flextensor_amd.nn import batch_gemm as op_batch_gemm
+    nb, M, K, N = 3, 40, 48, 72
+    for ta, tb in ((True, False), (True, True), (False, True)):
+        def wrap(nb, M, K, N, ta=ta, tb=tb):
+            A = placeholder((nb, K, M) if ta else (nb, M, K), name="A")
+            B = placeholder((nb, N, K) if tb else (nb, K, N), name="B")
+            C = op_batch_gemm(A, B, transposeA=ta, transposeB=tb)
+            return [C.op], [A, B, C]
+        name = "batch_gemm_%d%d" % (ta, tb)
+        register(wrap, "gemm", name, (nb, M, K, N), "rocm", 0)
+        key = key_of("gemm", name, (nb, M, K, N))
+        ops, bufs = wrap(nb, M, K, N)
+        a, b = seeded_inputs(bufs, seed=5)
+        ref = np.stack([oracle.gemm_f32_c(a[i], b[i], transA=ta, transB=tb) for i in range(nb)])
+        a64 = a.astype(np.float64).transpose(0, 2, 1) if ta else a.astype(np.float64)
+        b64 = b.astype(np.float64).transpose(0, 2, 1) if tb else b.astype(np.float64)
+        assert rel(ref, np.matmul(a64, b64)) <= TOL
+        for cfg in (Config([], None), Config([gcfg(M, N, K, 1, 1, 2, 1, 16, 16, st=3)], None)):
+            out = run_plan(key, cfg, [a, b])
+            assert rel(out, ref) <= TOL, (ta, tb)
+        dev = [torch.from_numpy(x).cuda() for x in (a, b)]
+        out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+        run_default_schedule(ops, dev + [out], stream=current_stream())
+        torch.cuda.synchronize()
+        assert rel(out.cpu().numpy(), ref) <= TOL
+
+
 def test_gemm_transpose_b_vs_oracle(oracle):
     def wrap(M, K, N):
         A = placeholder((M, K), name="A")
@@ -756,6 +785,10 @@ def test_depthwise_shuffled_halo_vs_oracle(oracle, args, th, waves):
     ones = np.ones_like(x)
     out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, 4, waves), special=[[0], [1]]), [ones, w])
     assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
+    # several patches per lane (lane_items), requested up front: shuffled halo, loaded halo, scalar path
+    for items, shfl, tw in ((3, 1, 4), (2, 0, 4), (4, 0, 2)):
+        out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, th, tw, waves), special=[[1], [shfl], [0], [items]]), [x, w])
+        assert rel(out, ref) <= TOL, (items, shfl, tw)
 
 
 @pytest.mark.parametrize("args,planes,waves", [

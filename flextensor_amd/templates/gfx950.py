@@ -401,8 +401,6 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
             bv, bpad = 4, 0   # B in 16-byte chunks too: unpadded rows, columns swizzled by k
         elif view.mode != 2:
             bv = 1            # B goes one float per lane
-        if apad < 0 and (bk & (bk - 1)) != 0:
-            apad = 0          # rows land contiguously: unpadded when the swizzle is not available
         if av != 4 or apad > 0 or (bm * bk // 4) % 64:
             raise InvalidConfig("direct-to-LDS tiles need 16-byte A chunks in whole wavefronts and unpadded A rows")
         if view.mode == 2 and (bv != 4 or (bn * bk // 4) % 64):
@@ -415,8 +413,6 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
             if bpad != 0 or (bn * bk) % 64:
                 raise InvalidConfig("direct-to-LDS tiles with rows that are not multiples of 64 floats need "
                                     "unpadded B rows and whole wavefronts of floats per tile")
-    if apad < 0 and (bk & (bk - 1)) != 0:
-        apad = 4              # the chunk swizzle needs a power-of-two row
     sa = bk + max(apad, 0)
     if view.mode == 2:
         lds_b = bn * sa

@@ -277,6 +277,10 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     (96, 144, 128, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=72, st=5), [0, 0]),               # partial last round of chunks
     (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=5), [0, 0]),               # B in swizzled 16-byte chunks, ragged
     (256, 256, 512, dict(wm=2, rm=2, wn=2, rn=4, mf=16, bk=32, st=5), [-1, -1]),            # same, 128-wide tile
+    (96, 144, 128, dict(wm=1, rm=1, wn=1, rn=2, mf=32, bk=72, st=5), [-1, 0]),              # 18 chunks a row: XOR of the low chunk bit
+    (128, 288, 128, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=48, st=5), [-1, -1]),            # 12 chunks a row: XOR of two bits
+    (128, 288, 64, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=144, st=5), [-1, 0]),             # 36 chunks a row
+    (128, 240, 64, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=40, st=5), [-1, 0]),              # 10 chunks a row
     # three and four buffers: two and three tiles requested ahead
     (256, 512, 256, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=64, st=6), [-1, -1]),
     (256, 512, 256, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=7), [-1, -1]),
@@ -300,6 +304,26 @@ def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
     assert rel(out, oracle.gemm_np(a, b)) <= TOL
 
 
+@pytest.mark.parametrize("M,K,N,kn", [
+    (128, 288, 128, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=48, st=3)),     # 12 chunks a row
+    (200, 216, 136, dict(wm=2, rm=1, wn=1, rn=2, mf=32, bk=72, st=2)),     # 18 chunks, ragged M and N
+    (128, 240, 64, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=40, st=4)),      # 10 chunks
+])
+def test_gemm_f32_swizzled_rows_of_any_even_length(oracle, M, K, N, kn):
+    """lds_pad -1 on the register-staged pipelines: unpadded A rows whose chunk
+    index is XOR-ed by the row, also when the row is not a power of two long."""
+    register(gemm, "gemm", "gemm", (M, K, N), "rocm", 0)
+    key = key_of("gemm", "gemm", (M, K, N))
+    ops, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=M + N)
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[0]], [[-1, -1]]
+    s, _ = schedule_with_config(key, Config([gcfg(M, N, K, **kn)], g))
+    assert s.specs[-1].defines["APAD"] == -1
+    out = run_plan(key, Config([gcfg(M, N, K, **kn)], g), [a, b])
+    assert rel(out, oracle.gemm_np(a, b)) <= TOL
+
+
 def test_gemm_transpose_b_direct_to_lds(oracle):
     def wrap(M, K, N):
         A = placeholder((M, K), name="A")
@@ -320,6 +344,9 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
 @pytest.mark.parametrize("args,kn,pad", [
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=16, st=5), [-1, 8]),
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=5), [0, 0]),     # groups, hoisted gather
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=5), [-1, 0]),    # same, rows of 18 chunks swizzled
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=48, sk=4, wk=1, st=5), [-1, 0]),  # 12 chunks, 4 k-groups
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=144, st=5, ks=1), [-1, 0]),   # 36 chunks, K streaming
     ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=2, wn=4, rn=1, mf=16, bk=16, st=5), [-1, 4]),     # stride 2, K tail
     ((3, 8, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=16, st=5, ks=1), [-1, 4]),   # dilation, K streaming
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, 8]),      # 1x1, N=392

@@ -22,6 +22,13 @@
 // border stands for the padding, and writes the outputs in the same order.
 // It needs a same-size 3x3 / stride 1 / dilation 1 / padding 1 layer with
 // FACT == 1 and rows that are multiples of four floats.
+// WX > 0 selects the row-exchange variant for the same kind of layer: a
+// wavefront owns WXR * WX consecutive rows of one plane (WXR whole rows per
+// load instruction, WX 16-byte chunks per lane), loads each chunk once, in
+// copy order, all loads issued before anything else, and passes the rows
+// above and below between lanes through a wavefront-private LDS window: no
+// barrier, no halo re-reads from memory except the one row either side of
+// the span; the padding rows arrive as the zeros of out-of-range loads.
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
 // STRH/STRW, PADH/PADW, DILH/DILW (rows / columns), FACT, CP x CQ output.
 
@@ -46,6 +53,11 @@
 #define LDSP FT_LDSP
 #else
 #define LDSP 0
+#endif
+#ifdef FT_WX
+#define WX FT_WX          /* chunks per lane of the row-exchange variant */
+#else
+#define WX 0
 #endif
 #define CB FT_CB
 #define CC FT_CC
@@ -171,6 +183,108 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #else
         O4[(size_t)plane * PLANE4 + rem] = acc;
 #endif
+    }
+}
+#elif WX > 0
+#if !(STRH == 1 && STRW == 1 && DILH == 1 && DILW == 1 && CR == 3 && CS == 3 && PADH == 1 && PADW == 1 && CP == CH && CQ == CW && CW % 4 == 0 && FACT == 1)
+#error "the row-exchange variant needs a same-size 3x3 stride-1 pad-1 layer, FACT 1, CW % 4 == 0"
+#endif
+#define Q4 (CW / 4)                  /* 128-bit chunks per row */
+#define PLANE4 (CH * Q4)             /* ... per plane */
+#define NCH (PLANES * PLANE4)        /* ... of the tensor */
+#define RPI FT_WXR                   /* whole rows one load instruction of a wavefront covers */
+#define LPW (RPI * Q4)               /* lanes that carry work */
+#define ROWS (RPI * WX)              /* rows one wavefront owns */
+#define SPP ((CH + ROWS - 1) / ROWS) /* wavefronts per plane */
+#define WIN ((ROWS + 2) * Q4)        /* chunks of a wavefront's LDS window: row above, rows, row below */
+#if LPW > 64 || LPW < 1 || 2 * Q4 > 64
+#error "row exchange: whole rows per instruction, rows of at most 128 floats"
+#endif
+#define OOB 0x80000000u
+#define X_BYTES (NCH * 16)
+#define LD_AUX (NT_LOAD ? 2 : 0)     /* bit 1 of the cache policy operand: non-temporal */
+#define ST_AUX (NT_STORE ? 2 : 0)
+
+extern "C" __global__ __launch_bounds__(NT)
+void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
+                   float* __restrict__ O)
+{
+    /* window chunk ro * Q4 + col of a wavefront holds (row r0 - 1 + ro, chunk col) of its plane */
+    __shared__ __attribute__((aligned(16))) float sx[(NT / 64) * WIN * 4];
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, X_BYTES, 0x00020000);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wid = blockIdx.x * (NT / 64) + wave;              /* wavefront-uniform from here on */
+    const int plane = wid / SPP;
+    const int r0 = (wid - plane * SPP) * ROWS;                  /* first row of the span */
+    const int lr = lane / Q4, col = lane - lr * Q4;
+    float* win = &sx[wave * WIN * 4];
+    const bool plane_ok = plane < PLANES;
+
+    /* ---- every load first: the rows in copy order, then the rows above and below ---- */
+    f32x4 v[WX];
+    unsigned vo[WX];
+#pragma unroll
+    for (int i = 0; i < WX; ++i) {
+        const int row = r0 + i * RPI + lr;
+        const bool ok = plane_ok && lane < LPW && row < CH;
+        vo[i] = ok ? (unsigned)(plane * PLANE4 + row * Q4 + col) * 16u : OOB;
+        v[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo[i], 0, LD_AUX));
+    }
+    /* lanes 0 .. Q4-1 fetch the row above the span, the next Q4 lanes the row below; rows
+     * outside the plane are the padding and read as zero, like everything an idle lane asks for */
+    const int hrow = lane < Q4 ? r0 - 1 : r0 + ROWS;
+    const int hcol = lane < Q4 ? lane : lane - Q4;
+    const bool hok = plane_ok && lane < 2 * Q4 && hrow >= 0 && hrow < CH;
+    const f32x4 hv = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+        rx, (int)(hok ? (unsigned)(plane * PLANE4 + hrow * Q4 + hcol) * 16u : OOB), 0, LD_AUX));
+    /* the plane's kernel: wavefront-uniform, so scalar loads */
+    const int ch = __builtin_amdgcn_readfirstlane(plane_ok ? plane % CC : 0);     /* kernels repeat per batch entry */
+    float w[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+        w[t] = Wt[ch * 9 + t];
+
+    /* ---- rows change lanes through the window -------------------------------- */
+    if (lane < LPW) {
+#pragma unroll
+        for (int i = 0; i < WX; ++i)
+            *reinterpret_cast<f32x4*>(&win[((1 + i * RPI) * Q4 + lane) * 4]) = v[i];
+    }
+    if (lane < 2 * Q4)
+        *reinterpret_cast<f32x4*>(&win[(lane < Q4 ? lane : (ROWS + 1) * Q4 + lane - Q4) * 4]) = hv;
+    /* LDS operations of one wavefront complete in order; the fences keep the compiler from
+     * moving the reads below above the writes of the other lanes */
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    const bool left = col == 0, right = col == Q4 - 1;
+#pragma unroll
+    for (int i = 0; i < WX; ++i) {
+        const float* mid = &win[((1 + i * RPI) * Q4 + (lane < LPW ? lane : 0)) * 4];   /* idle lanes stay inside the window */
+        f32x4 acc = (f32x4)(0.0f);
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const float* base = mid + (r - 1) * Q4 * 4;
+            const f32x4 m = r == 1 ? v[i] : *reinterpret_cast<const f32x4*>(base);
+            /* the columns left and right of the four come from the neighbouring lanes' vectors
+             * (DPP wavefront shifts by one lane); at the ends of a row they are the padding */
+            /* (both shifts run in every lane, outside the selects: a lane switched off by a
+             * branch could not be read by its neighbour) */
+            const int from_below = __builtin_amdgcn_update_dpp(0, __float_as_int(m[3]), 0x138, 0xf, 0xf, false);
+            const int from_above = __builtin_amdgcn_update_dpp(0, __float_as_int(m[0]), 0x130, 0xf, 0xf, false);
+            const float lf = left ? 0.0f : __int_as_float(from_below);
+            const float rt = right ? 0.0f : __int_as_float(from_above);
+            const float in[6] = {lf, m[0], m[1], m[2], m[3], rt};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+                    acc[c] += in[c + t] * w[r * 3 + t];
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), ro, (int)vo[i], 0, ST_AUX);
     }
 }
 #else

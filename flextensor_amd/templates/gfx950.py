@@ -241,6 +241,7 @@ SPECIAL_DEFAULTS = {
     "halo_shfl": [0],
     "lds_planes": [0],
     "lane_items": [1],
+    "row_exchange": [0],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -263,7 +264,7 @@ def special_knobs(kind):
         return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]],
-                "lane_items": [[1], [2], [3], [4], [6], [8]]}
+                "lane_items": [[1], [2], [3], [4], [6], [8]], "row_exchange": [[0], [1], [2], [3], [4]]}
     return {}
 
 
@@ -547,6 +548,30 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
                  CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=1, CP=p, CQ=q, **steps)
         return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(b * cout, ldsp), 1, 1),
                            (nt, 1, 1),
+                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
+    wx = int(_special(special, "row_exchange")[0])
+    if wx:
+        # row-exchange variant: a wavefront owns rpi * wx rows of one plane (rpi whole rows per load
+        # instruction), loads each 16-byte chunk once and passes rows between lanes through its own
+        # LDS window; the lane patch knobs do not apply
+        if not (st_h == st_w == 1 and dl_h == dl_w == 1 and r_ext == 3 and s_ext == 3 and pad_h == pad_w == 1
+                and p == h and q == w and w % 4 == 0 and a["factor"] == 1):
+            raise InvalidConfig("row exchange needs a same-size 3x3 stride-1 pad-1 layer with rows of whole vectors")
+        q4 = w // 4
+        if wx < 1 or wx > 8 or 2 * q4 > 64:
+            raise InvalidConfig("row exchange: 1 .. 8 chunks per lane, rows of at most 128 floats")
+        # rows per instruction: as many as fit 64 lanes, fewer when that makes the spans tile the plane
+        rpi_max = min(64 // q4, h)
+        rpi = max([r for r in range(1, rpi_max + 1) if h % (r * wx) == 0] or [0])
+        if rpi * 4 < rpi_max * 3:
+            rpi = rpi_max         # too few lanes would carry work: ragged last span instead
+        rows = rpi * wx
+        if waves * (rows + 2) * q4 * 16 > LDS_BYTES:
+            raise InvalidConfig("row-exchange windows do not fit the LDS")
+        D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=0, WX=wx, WXR=rpi,
+                 CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=1, CP=p, CQ=q, **steps)
+        return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D,
+                           (ceil_div(b * cout * ceil_div(h, rows), waves), 1, 1), (nt, 1, 1),
                            [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
     shfl = int(_special(special, "halo_shfl")[0])
     tiles_w = ceil_div(q, tw)

@@ -818,6 +818,43 @@ def test_depthwise_shuffled_halo_vs_oracle(oracle, args, th, waves):
         assert rel(out, ref) <= TOL, (items, shfl, tw)
 
 
+@pytest.mark.parametrize("args,chunks,waves,rows_per_load", [
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 2, 4, 7),     # 14 rows per wavefront: two spans tile a plane
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 4, 2, 7),     # a whole plane per wavefront: every halo row is padding
+    ((2, 16, 28, 28, 1, 3, 1, 1, 1), 3, 1, 9),     # 27 rows + a ragged span of one row
+    ((1, 5, 8, 12, 1, 3, 1, 1, 1), 1, 1, 8),       # 3 chunks per row, 24 of 64 lanes busy; 5 planes
+    ((3, 7, 16, 64, 1, 3, 1, 1, 1), 2, 2, 4),      # 16 chunks per row; 21 planes x 2 spans on 2-wavefront workgroups
+    ((2, 3, 7, 4, 1, 3, 1, 1, 1), 8, 4, 7),        # one chunk per row: every chunk is left and right edge; more rows than the plane
+    ((1, 2, 5, 128, 1, 3, 1, 1, 1), 3, 1, 2),      # 32 chunks per row: the two halo rows take all 64 lanes
+])
+def test_depthwise_row_exchange_vs_oracle(oracle, args, chunks, waves, rows_per_load):
+    """Rows pass between lanes through a wavefront-private LDS window; every chunk is loaded once."""
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
+    b_, co, p, q = ref.shape
+    for nt_store in (0, 1, 3):
+        cfgs = conv_cfgs(dcfg(b_, co, p, q, 1, 4, waves), special=[[nt_store], [0], [0], [1], [chunks]])
+        s, _ = schedule_with_config(key, cfgs)
+        assert s.specs[-1].defines["WX"] == chunks and s.specs[-1].defines["WXR"] == rows_per_load
+        out = run_plan(key, cfgs, [x, w])
+        assert rel(out, ref) <= TOL, nt_store
+    # borders: a constant image must give border sums with missing taps
+    ones = np.ones_like(x)
+    out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, 1, 4, waves), special=[[0], [0], [0], [1], [chunks]]), [ones, w])
+    assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
+    # a layer it does not fit is refused, not mis-computed
+    for bad in ((1, 4, 9, 20, 2, 3, 1, 1, 1), (1, 4, 9, 20, 1, 3, 2, 1, 1), (1, 4, 9, 18, 1, 3, 1, 1, 1)):   # factor 2; stride 2; ragged rows
+        register(depthwise_conv2d, "conv2d", "depthwise", bad, "rocm", 0)
+        bo = oracle.depthwise_nchw_np(np.zeros((bad[0], bad[1], bad[2], bad[3]), np.float32),
+                                      np.zeros((bad[1], bad[4], 3, 3), np.float32), bad[6], bad[7], bad[8]).shape
+        with pytest.raises(Exception):
+            schedule_with_config(key_of("conv2d", "depthwise", bad),
+                                 conv_cfgs(dcfg(bo[0], bo[1], bo[2], bo[3], 1, 4, 1), special=[[0], [0], [0], [1], [2]]))
+
+
 @pytest.mark.parametrize("args,planes,waves", [
     ((2, 16, 28, 28, 1, 3, 1, 1, 1), 4, 4),
     ((1, 5, 8, 12, 1, 3, 1, 1, 1), 2, 1),         # 5 planes, 2 per workgroup: the last workgroup is half empty

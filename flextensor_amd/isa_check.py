@@ -8,7 +8,14 @@ workspace slot (a device-scope store, ``sc1``) to the next arrival count (a
 with ``vmcnt(0)``) and then passes an ``s_barrier``; neither a barrier nor a
 workgroup-scope fence waits for vector stores by itself.
 
-The hardware does not interlock this case; the compiler pads it with s_nop,
+3. Lane shifts under a narrowed execution mask: a DPP instruction reads a
+neighbouring lane's register, and a lane that a divergent branch has switched
+off cannot be read (the reader keeps its old value). The compiler is free to
+sink a shift into the arm of a select; the depthwise kernels therefore compute
+their shifts before any select, and this check looks for a DPP instruction
+between an ``s_and_saveexec`` and the instruction that restores ``exec``.
+
+For 1: the hardware does not interlock this case; the compiler pads it with s_nop,
 but its padding follows the control-flow graph with a visited set per block
 and can lose a short path. This module rebuilds the graph from the assembly
 text and walks every path forward from each MFMA for the required number of
@@ -181,6 +188,37 @@ def find_unordered_arrivals(asm_text, kernel):
     return found, insts
 
 
+NARROWS = re.compile(r"^s_(and|andn2|xor)_saveexec_b64$")
+
+
+def _restores_exec(name, ops):
+    """exec is whole again: or-ed with the saved mask, or re-loaded."""
+    return name in ("s_or_b64", "s_mov_b64", "s_or_saveexec_b64") and re.match(r"\s*exec\b", ops) is not None
+
+
+def find_masked_lane_shifts(asm_text, kernel):
+    """[(mask instruction index, DPP instruction index)] for DPP instructions that control
+    can reach from an instruction that narrows exec before exec is restored."""
+    insts, labels = parse(asm_text, kernel)
+    found = []
+    for i, (name, ops) in enumerate(insts):
+        if not NARROWS.match(name):
+            continue
+        stack, seen = list(_successors(insts, labels, i)), set()
+        while stack:
+            j = stack.pop()
+            if j in seen:
+                continue
+            seen.add(j)
+            jn, jo = insts[j]
+            if _restores_exec(jn, jo):
+                continue
+            if jn.endswith("_dpp"):
+                found.append((i, j))
+            stack.extend(_successors(insts, labels, j))
+    return found, insts
+
+
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
@@ -201,11 +239,16 @@ def assembly_of(spec, workdir=None):
 
 
 def check_plan(plan):
-    """[(kernel, first instruction, second instruction, detail)] over the MFMA kernels of a plan:
-    early reads of MFMA results (detail = issue slots between) and arrival counts of the
-    K-streaming exchange that do not wait for the slot stores (detail = "arrival")."""
+    """[(kernel, first instruction, second instruction, detail)] over the kernels of a plan:
+    early reads of MFMA results (detail = issue slots between), arrival counts of the
+    K-streaming exchange that do not wait for the slot stores (detail = "arrival"), and in
+    the depthwise kernels DPP lane shifts under a narrowed exec mask (detail = "masked shift")."""
     out = []
     for spec in plan.specs:
+        if spec.kernel == "depthwise_f32":
+            found, insts = find_masked_lane_shifts(assembly_of(spec), spec.kernel)
+            out.extend((spec.kernel, insts[i], insts[j], "masked shift") for i, j in found)
+            continue
         if spec.kernel not in ("igemm_f32", "gemm_i8"):
             continue
         text = assembly_of(spec)
@@ -236,6 +279,8 @@ def main(argv):
             bad += 1
             if used == "arrival":
                 print("UNORDERED ARRIVAL %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
+            elif used == "masked shift":
+                print("LANE SHIFT UNDER A NARROWED EXEC MASK %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
             else:
                 print("EARLY READ %s %s: %s %s -> %s %s after %d slots" % ((key, kernel) + mfma + reader + (used,)))
     print("%d plans checked, %d findings" % (len(seen), bad))

@@ -165,3 +165,43 @@ def test_k_streaming_arrivals_wait_for_the_slot_stores(tmp_path):
         assert re.search(r"global_store_dword.*sc1", text) and "global_atomic_add" in text
         found, insts = isa_hazards.find_unordered_arrivals(text, spec.kernel)
         assert found == [], [(insts[i], insts[j]) for i, j in found[:3]]
+
+
+MASKED = """k:
+\tv_cmp_ne_u32_e32 vcc, 0, v12
+\tv_mov_b32_e32 v23, 0
+%s.LBB0_2:
+\ts_or_b64 exec, exec, s[2:3]
+\tv_mov_b32_dpp v24, v7 wave_shl:1 row_mask:0xf bank_mask:0xf
+\ts_endpgm
+.Lfunc_end0:
+"""
+
+
+def test_lane_shift_checker_flags_a_shift_behind_a_narrowed_mask():
+    branchy = ("\ts_and_saveexec_b64 s[2:3], vcc\n\ts_cbranch_execz .LBB0_2\n"
+               "\tv_mov_b32_dpp v23, v11 wave_shr:1 row_mask:0xf bank_mask:0xf\n")
+    found, insts = isa_hazards.find_masked_lane_shifts(MASKED % branchy, "k")
+    # the shift inside the branch is found; the one after exec is whole again is not
+    assert [(insts[i][0], insts[j][1].split()[0]) for i, j in found] == [("s_and_saveexec_b64", "v23,")]
+    plain = "\tv_mov_b32_dpp v23, v11 wave_shr:1 row_mask:0xf bank_mask:0xf\n\tv_cndmask_b32_e32 v23, 0, v23, vcc\n"
+    found, _ = isa_hazards.find_masked_lane_shifts(MASKED % plain, "k")
+    assert found == []
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+@pytest.mark.parametrize("special", [[[1], [0], [0], [1], [2]],      # row exchange (the shipped variant)
+                                     [[1], [0], [0], [1], [3]],      # ragged last span
+                                     [[1], [1], [0], [1], [0]],      # direct kernel, shuffled halo
+                                     [[1], [1], [0], [3], [0]]])     # the same, three patches per lane
+def test_depthwise_lane_shifts_run_with_every_lane_switched_on(special):
+    key = "conv2d_depthwise_(8, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)"
+    c = {k: [] for k in KEYS}
+    c["spatial"] = [[8, 1, 1, 1], [512, 1, 1, 1], [28, 1, 1, 1], [7, 1, 1, 4]]
+    c["fuse"] = [[4]]
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[1, 0]], special
+    plan, _ = schedule_with_config(key, Config([{k: [] for k in KEYS}, c], g))
+    text = isa_hazards.assembly_of(plan.specs[-1])
+    assert "_dpp" in text, "the kernel is expected to shift lanes with DPP"
+    assert isa_hazards.check_plan(plan) == []

@@ -195,7 +195,7 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7, 8] if i8 else [1, 2, 3, 4, 5, 6, 7], explicit=True),
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7, 8], explicit=True),
                        "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
@@ -300,11 +300,14 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     (gm, wm, rm, mfm), (gn, wn, rn, mfn) = [list(map(int, x)) for x in sp]
     splitk, kiters, bk = [int(x) for x in rd[0]]
     depth = int((config.get("unroll") or [[2, 1]])[0][0])
-    if depth not in PIPELINE or (depth == 8 and view.dtype != "int8"):
+    if depth not in PIPELINE:
         raise InvalidConfig("pipeline depth %d is not available" % depth)
     stages, pd = PIPELINE[depth]
-    if view.dtype != "int8" and depth >= 6:
+    if view.dtype != "int8" and depth in (6, 7):
         stages = depth - 3        # fp32: 6 and 7 = tiles straight into LDS with three and four buffers
+    # fp32 depth 8: as 5 (two buffers), and the first operands of the next tile are read from LDS
+    # right behind the barrier, ahead of the last MFMAs of the current tile
+    frag_prefetch = view.dtype != "int8" and depth == 8
     group_m = int((config.get("fuse") or [[4]])[0][0])
     ro = list((config.get("reorder") or [[1, 0]])[0]) + [0, 0]
     xcd, in_wg, stream_k = int(ro[0]), int(ro[1]), int(ro[2])
@@ -449,6 +452,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         D.update(TA=1)
     if dtl:
         D.update(DTL=1)
+    if frag_prefetch:
+        D.update(FPF=1)
     specs = []
     if view.mode == 1:
         conv = dict(view.conv)

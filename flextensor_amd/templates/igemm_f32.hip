@@ -103,6 +103,11 @@
 #else
 #define DTL 0
 #endif
+#ifdef FT_FPF
+#define FPF FT_FPF          /* 1: first operands of the next tile read ahead of the last MFMAs of this one */
+#else
+#define FPF 0
+#endif
 #ifdef FT_COLOUT
 #define COLOUT FT_COLOUT
 #else
@@ -753,72 +758,86 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         for (int j = 0; j < REP_N; ++j)
             acc[i][j] = (acc_t)(0.0f);
 
-    auto compute = [&](int buf) {
-        const int arow = wm * REP_M * MFMA + li;   /* + i*MFMA: SWZ is the same when MFMA % 16 == 0 */
-        const float* as = &As[buf][arow * SA];
-        int acls[SWZ_CLASSES];
+    /* ---- MFMA operands: LDS -> registers -> matrix core ------------------ */
+    /* lane constants of the fragment reads (the same for every tile and buffer) */
+    const int arow = wm * REP_M * MFMA + li;   /* + i*MFMA: SWZ is the same when MFMA % 16 == 0 */
+    int acls[SWZ_CLASSES];
 #pragma unroll
-        for (int c = 0; c < SWZ_CLASSES; ++c)
-            acls[c] = ((c * KL + lg) ^ SWZ(arow)) << 2;
+    for (int c = 0; c < SWZ_CLASSES; ++c)
+        acls[c] = ((c * KL + lg) ^ SWZ(arow)) << 2;
 #if MODE == 2
-        const int brow = wn * REP_N * MFMA + li;
-        const float* bs = &Bs[buf][brow * SB];
-        int bcls[SWZ_CLASSES];
+    const int brow = wn * REP_N * MFMA + li;
+    int bcls[SWZ_CLASSES];
 #pragma unroll
-        for (int c = 0; c < SWZ_CLASSES; ++c)
-            bcls[c] = ((c * KL + lg) ^ SWZ(brow)) << 2;
+    for (int c = 0; c < SWZ_CLASSES; ++c)
+        bcls[c] = ((c * KL + lg) ^ SWZ(brow)) << 2;
 #elif defined(BSWZ)
-        /* physical column of logical column n in row kb + 4*lg + s: n ^ (lane part) ^ (kb part) */
-        const float* bs = &Bs[buf][(4 * lg) * SB];
-        int bcolx[REP_N];
+    /* physical column of logical column n in row kb + 4*lg + s: n ^ (lane part) ^ (kb part) */
+    int bcolx[REP_N];
 #pragma unroll
-        for (int j = 0; j < REP_N; ++j)
-            bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ (MFMA == 16 ? (lg << 4) : (lg << 5));
+    for (int j = 0; j < REP_N; ++j)
+        bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ (MFMA == 16 ? (lg << 4) : (lg << 5));
 #elif defined(BSWZ1)
-        /* logical (kb + 4*lg + s, n) sits at row kb + 4*lg + (s ^ BSW_R(lg)), column n ^ BSW_C(lg) */
+    /* logical (kb + 4*lg + s, n) sits at row kb + 4*lg + (s ^ BSW_R(lg)), column n ^ BSW_C(lg) */
+    int bcolx[REP_N], browx[4];
+#pragma unroll
+    for (int j = 0; j < REP_N; ++j)
+        bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ BSW_C(lg);
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+        browx[s] = (s ^ BSW_R(lg)) * SB;
+#endif
+    /* the operands of the k block [kb, kb + KBLK) of the tile in LDS buffer buf:
+     * a[i] = four k values of row block i, b[s][j] = k value s of column block j */
+    auto read_block = [&](int buf, int kb, f32x4 (&a)[REP_M], float (&b)[4][REP_N]) {
+        const float* as = &As[buf][arow * SA];
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+            a[i] = *reinterpret_cast<const f32x4*>(as + i * MFMA * SA + SWZ_HI(kb) + acls[SWZ_CLS(kb)]);
+#if MODE == 2
+        const float* bs = &Bs[buf][brow * SB];
+#pragma unroll
+        for (int j = 0; j < REP_N; ++j) {
+            const f32x4 b4 = *reinterpret_cast<const f32x4*>(bs + j * MFMA * SB + SWZ_HI(kb) + bcls[SWZ_CLS(kb)]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                b[s][j] = b4[s];
+        }
+#else
+#if defined(BSWZ) || defined(BSWZ1)
         const float* bs = &Bs[buf][(4 * lg) * SB];
-        int bcolx[REP_N], browx[4];
-#pragma unroll
-        for (int j = 0; j < REP_N; ++j)
-            bcolx[j] = (wn * REP_N * MFMA + j * MFMA + li) ^ BSW_C(lg);
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-            browx[s] = (s ^ BSW_R(lg)) * SB;
 #else
         const float* bs = &Bs[buf][(4 * lg) * SB + wn * REP_N * MFMA + li];
 #endif
 #pragma unroll
-        for (int kb = 0; kb < BK; kb += KBLK) {
-            f32x4 a[REP_M];
-#pragma unroll
-            for (int i = 0; i < REP_M; ++i)
-                a[i] = *reinterpret_cast<const f32x4*>(as + i * MFMA * SA + SWZ_HI(kb) + acls[SWZ_CLS(kb)]);
-#if MODE == 2
-            f32x4 b4[REP_N];
+        for (int s = 0; s < 4; ++s)
 #pragma unroll
             for (int j = 0; j < REP_N; ++j)
-                b4[j] = *reinterpret_cast<const f32x4*>(bs + j * MFMA * SB + SWZ_HI(kb) + bcls[SWZ_CLS(kb)]);
+#if defined(BSWZ)
+                b[s][j] = bs[(kb + s) * SB + (bcolx[j] ^ (MFMA == 16 ? 0 : (((kb >> 2) & 1) << 5)))];
+#elif defined(BSWZ1)
+                b[s][j] = bs[kb * SB + browx[s] + bcolx[j]];
+#else
+                b[s][j] = bs[(kb + s) * SB + j * MFMA];
 #endif
+#endif
+    };
+    auto mfma_block = [&](const f32x4 (&a)[REP_M], const float (&b)[4][REP_N]) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                float b[REP_N];
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i)
 #pragma unroll
                 for (int j = 0; j < REP_N; ++j)
-#if MODE == 2
-                    b[j] = b4[j][s];
-#elif defined(BSWZ)
-                    b[j] = bs[(kb + s) * SB + (bcolx[j] ^ (MFMA == 16 ? 0 : (((kb >> 2) & 1) << 5)))];
-#elif defined(BSWZ1)
-                    b[j] = bs[kb * SB + browx[s] + bcolx[j]];
-#else
-                    b[j] = bs[(kb + s) * SB + j * MFMA];
-#endif
+                    acc[i][j] = MFMA_OP(a[i][s], b[s][j], acc[i][j]);
+    };
+    auto compute = [&](int buf) {
 #pragma unroll
-                for (int i = 0; i < REP_M; ++i)
-#pragma unroll
-                    for (int j = 0; j < REP_N; ++j)
-                        acc[i][j] = MFMA_OP(a[i][s], b[j], acc[i][j]);
-            }
+        for (int kb = 0; kb < BK; kb += KBLK) {
+            f32x4 a[REP_M];
+            float b[4][REP_N];
+            read_block(buf, kb, a, b);
+            mfma_block(a, b);
         }
     };
 
@@ -951,6 +970,46 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             __syncthreads();
             cur = (cur + 1 == STAGES) ? 0 : cur + 1;
             nxt = (nxt + 1 == STAGES) ? 0 : nxt + 1;
+        }
+    }
+#elif DTL && FPF
+    /* Two buffers, and the operands of a tile's first k block are read right behind the
+     * barrier that ends the tile before it, ahead of that tile's last MFMAs: the LDS
+     * latency of the first reads, which every wavefront of the workgroup would otherwise
+     * sit out together after each barrier, hides behind matrix work. The barrier stands
+     * before the last k block's MFMAs; all reads of the current buffer have returned by
+     * then (lgkmcnt(0)), so the next iteration may overwrite it. */
+    {
+        f32x4 pa[REP_M];
+        float pb[4][REP_N];
+        read_block(0, 0, pa, pb);
+        for (int kt = 0; kt < nk; ++kt) {
+            const int cur = kt & 1;
+            if (kt + 1 < nk) dma_tile(kt + 1, cur ^ 1);      /* lands while tile kt is multiplied */
+            f32x4 a[2][REP_M], na[REP_M];
+            float b[2][4][REP_N], nb[4][REP_N];
+#pragma unroll
+            for (int blk = 0; blk < BK / KBLK; ++blk) {
+                if (blk + 1 < BK / KBLK) read_block(cur, (blk + 1) * KBLK, a[(blk + 1) & 1], b[(blk + 1) & 1]);
+                if (blk == BK / KBLK - 1) {
+                    __builtin_amdgcn_s_waitcnt(0x0070);      /* vmcnt(0), lgkmcnt(0) */
+                    __syncthreads();
+                    /* after the last tile this reads stale data that nothing uses */
+                    read_block(cur ^ 1, 0, na, nb);
+                }
+                /* the reads above are issued before the MFMAs below, which then hide their latency
+                 * (left alone, the scheduler puts each read right in front of its first use) */
+                __builtin_amdgcn_sched_barrier(0);
+                if (blk == 0) mfma_block(pa, pb);
+                else mfma_block(a[blk & 1], b[blk & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < REP_M; ++i) pa[i] = na[i];
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < REP_N; ++j) pb[s][j] = nb[s][j];
         }
     }
 #elif DTL

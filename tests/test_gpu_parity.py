@@ -288,6 +288,13 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16, st=6), [0, 0]),               # ragged, padded K, odd tile count
     (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=6, ks=1), [-1, -1]),      # with K streaming: segments of any length
     (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=7, ks=2), [-1, -1]),
+    # depth 8: two buffers, the next tile's first operands read behind the barrier, ahead of the last MFMAs
+    (256, 256, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=8), [-1, -1]),
+    (200, 136, 328, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=8, st=8), [0, 8]),               # one k block per tile, ragged, padded K
+    (256, 64, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=64, st=8), [-1, -1]),             # a single tile
+    (128, 288, 128, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=48, st=8), [-1, -1]),            # three k blocks per tile
+    (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=8, ks=1), [-1, -1]),      # K streaming: segments of any length
+    (256, 512, 256, dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32, sk=4, wk=1, st=8), [-1, -1]),  # four k-groups in the workgroup
 ])
 def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
     """Pipeline depths 5 to 7: tiles travel global -> LDS without staging registers."""
@@ -368,6 +375,12 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     # rows that neither divide nor are multiples of 64 floats: the tile lands flat, not permuted
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=5, mf=16, bk=32, st=5), [-1, 0]),      # 80 floats, N=392
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=3, mf=16, bk=16, st=5), [0, 0]),     # 48 floats
+    # depth 8 (operands of the next tile read ahead of the last MFMAs)
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, st=8), [-1, 0]),    # groups, whole windows
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=144, st=8), [0, 0]),    # 16 columns, four tiles of 144
+    ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, st=8), [-1, 0]),      # 1x1, N=392
+    ((3, 8, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=16, st=8, ks=1), [-1, 4]),   # dilation, K tail, K streaming
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=144, st=8, ks=1), [-1, 0]),  # 36 chunks, K streaming
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)

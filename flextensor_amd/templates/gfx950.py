@@ -18,6 +18,7 @@ Operator kinds and the template each one lowers to:
 
 Meaning of the config keys: see flextensor_amd/space.py.
 """
+import json
 import os
 
 from ..space import (Space, SplitSpace, TileSplitSpace, LaneTileSpace, UnrollSpace, EnumSpace)
@@ -236,7 +237,9 @@ SPECIAL_DEFAULTS = {
     # BPAD -1 = the padding that spreads the k-groups of one MFMA operand read
     # over disjoint banks (4 floats for 16x16x4, 8 for 32x32x2).
     # int8: [PAD bytes / 4, unused]
-    "lds_pad": [4, -1],
+    # the default admits every pipeline depth (tiles straight into LDS need unpadded A rows), so
+    # that an operator search under the graph level's defaults can reach them
+    "lds_pad": [-1, -1],
     "nt_store": [0],
     "halo_shfl": [0],
     "lds_planes": [0],
@@ -259,9 +262,9 @@ def special_knobs(kind):
     """Enumerated knobs a task of this operator kind carries by default; they
     are attached with Task.set_specific_space and searched at graph level."""
     if kind in ("gemm", "conv2d_nchw", "batch_gemm", "col_gemm"):
-        return {"lds_pad": [[4, -1], [-1, -1], [4, 8], [4, 4], [0, 0], [8, -1]]}
+        return {"lds_pad": [[-1, -1], [4, -1], [4, 8], [4, 4], [0, 0], [8, -1], [-1, 0]]}
     if kind == "gemm_int8":
-        return {"lds_pad": [[4, 0], [-1, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
+        return {"lds_pad": [[-1, 0], [4, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]],
                 "lane_items": [[1], [2], [3], [4], [6], [8]], "row_exchange": [[0], [1], [2], [3], [4]]}
@@ -769,7 +772,7 @@ def seed_configs(op, limit=24):
                   ((4, 1, 16), (1, 1, 16)), ((4, 1, 16), (2, 1, 16)), ((2, 2, 16), (4, 1, 16)),
                   ((2, 1, 16), (4, 1, 16))]
         bks = [b for b in (144, 72, 64, 48, 32) if b in F32_BK]
-        depths, streams = [5, 3, 2, 1], [0, 1]
+        depths, streams = [8, 5, 3, 2, 1], [0, 1]
     def in_space(extent, t):
         # the tile space's own rules: no tile a smaller one covers as well, bounded edge waste
         size = t[1] * t[2] * t[3]
@@ -819,5 +822,28 @@ def seed_configs(op, limit=24):
         step = (len(lst) - 1) / float(max(n - 1, 1))
         return [lst[int(round(i * step))] for i in range(n)]
 
+    def spread_groups(first, lst, n):
+        """``first`` and n - 1 of ``lst``: the (tile, BK) groups are visited in turn, and each visit
+        of a group takes its next (depth, streaming) variant, starting at a variant that moves
+        with the group, so that every tile shape and every pipeline depth gets measured."""
+        if len(lst) + 1 <= n:
+            return [first] + lst
+        groups, index = [], {}
+        for c in lst:
+            gkey = json.dumps([c["spatial"], c["reduce"]])
+            if gkey not in index:
+                index[gkey] = len(groups)
+                groups.append([])
+            groups[index[gkey]].append(c)
+        picked, taken, k = [first], [0] * len(groups), 0
+        while len(picked) < n:
+            gi = k % len(groups)
+            g = groups[gi]
+            if taken[gi] < len(g):
+                picked.append(g[(taken[gi] + gi) % len(g)])
+                taken[gi] += 1
+            k += 1
+        return picked
+
     nsplit = min(len(split_seeds), limit // 3)
-    return spread(out, limit - nsplit) + spread(split_seeds, nsplit)
+    return spread_groups(out[0], out[1:], limit - nsplit) + spread(split_seeds, nsplit)

@@ -105,8 +105,15 @@ def test_lowering_rejects_bad_configs():
         _gemm_cfg([2, 2, 8, 32], [2, 2, 8, 32], [1, 64, 16]),     # 1024 accumulators
         _gemm_cfg([8, 8, 1, 16], [8, 8, 1, 16], [1, 64, 16]),     # 64 wavefronts
         _gemm_cfg([32, 2, 1, 16], [32, 2, 1, 16], [1, 128, 8]),   # BK < 16 with 16x16x4
-        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=5),
+        _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=9),   # no such pipeline depth
     ]
+    # tiles straight into LDS (depth 5) land in unpadded rows: a padded A tile is refused
+    dtl = _gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [1, 64, 16], stages=5)
+    assert schedule_with_config(GEMM, Config([dtl], None))[0].specs[0].defines["DTL"] == 1
+    padded = {k: [] for k in dtl}
+    padded["special"] = [[4, -1]]
+    with pytest.raises(gfx950.InvalidConfig):
+        schedule_with_config(GEMM, Config([dtl], padded))
     for cfg in bad:
         with pytest.raises(gfx950.InvalidConfig):
             schedule_with_config(GEMM, Config([cfg], None))

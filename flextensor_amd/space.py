@@ -218,12 +218,12 @@ class ReorderSpace(_RingSpace):
 
 
 class UnrollSpace(_RingSpace):
-    def __init__(self, steps, explicit=False):
+    def __init__(self, steps, explicit=False, extra=()):
         super(UnrollSpace, self).__init__()
         self.dim = 2
         self.steps = steps
         explicits = [1] if explicit else [0, 1]
-        self.static_entities = [[step, e] for step in steps for e in explicits]
+        self.static_entities = [[step, e] for step in steps for e in explicits] + [list(e) for e in extra]
         self.type_key = "unroll"
         self._finish()
 

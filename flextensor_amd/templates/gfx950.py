@@ -196,7 +196,8 @@ def _gemm_space(view):
     if rs.size == 0:
         raise InvalidConfig("K=%d has no admissible LDS tile extent" % view.K)
     space.add_subspace("split_k_0", rs, "reduce")
-    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7, 8], explicit=True),
+    space.add_subspace("unroll", UnrollSpace([1, 2, 3, 4, 5, 6, 7, 8], explicit=True,
+                                               extra=() if i8 else [[8, 2], [8, 4], [8, 6], [8, 8]]),
                        "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
@@ -311,6 +312,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     # fp32 depth 8: as 5 (two buffers), and the first operands of the next tile are read from LDS
     # right behind the barrier, ahead of the last MFMAs of the current tile
     frag_prefetch = view.dtype != "int8" and depth == 8
+    # with it, the second number of the unroll entry is the number of k blocks over which the
+    # loads of the next tile are spread (1 = all in front of the tile's first MFMAs)
+    load_spread = int((config.get("unroll") or [[2, 1]])[0][1]) if frag_prefetch else 1
     group_m = int((config.get("fuse") or [[4]])[0][0])
     ro = list((config.get("reorder") or [[1, 0]])[0]) + [0, 0]
     xcd, in_wg, stream_k = int(ro[0]), int(ro[1]), int(ro[2])
@@ -457,6 +461,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         D.update(DTL=1)
     if frag_prefetch:
         D.update(FPF=1)
+        if load_spread < 1 or (load_spread > 1 and load_spread > bk // kblk - 1):
+            raise InvalidConfig("the loads of the next tile spread over at most all but the last k block")
+        if load_spread > 1:
+            D.update(LSPREAD=load_spread)
     specs = []
     if view.mode == 1:
         conv = dict(view.conv)

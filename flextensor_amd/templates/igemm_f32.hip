@@ -108,6 +108,11 @@
 #else
 #define FPF 0
 #endif
+#ifdef FT_LSPREAD
+#define LSPREAD FT_LSPREAD  /* with FPF: k blocks over which the loads of the next tile are spread */
+#else
+#define LSPREAD 1
+#endif
 #ifdef FT_COLOUT
 #define COLOUT FT_COLOUT
 #else
@@ -869,10 +874,12 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                      :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
     };
-    auto dma_tile = [&](int kt, int buf) {
+    /* part p of np: the loads e of the tile with e mod np == p (A first, then B) */
+    auto dma_tile = [&](int kt, int buf, int part = 0, int nparts = 1) {
         const int k0 = kbase + kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
+            if (e % nparts != part) continue;
             unsigned vo = a_voff[e];
             if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
             if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))     /* whole wavefronts only */
@@ -881,6 +888,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
             if (!((B_CHUNKS % NT == 0) || (e * NT + wv * 64 < B_CHUNKS))) continue;
+            if ((EA + e) % nparts != part) continue;
 #if MODE == 2
             unsigned vo = b_voff[e];
             if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
@@ -985,11 +993,14 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         read_block(0, 0, pa, pb);
         for (int kt = 0; kt < nk; ++kt) {
             const int cur = kt & 1;
-            if (kt + 1 < nk) dma_tile(kt + 1, cur ^ 1);      /* lands while tile kt is multiplied */
             f32x4 a[2][REP_M], na[REP_M];
             float b[2][4][REP_N], nb[4][REP_N];
 #pragma unroll
             for (int blk = 0; blk < BK / KBLK; ++blk) {
+                /* the next tile's loads, in LSPREAD parts in front of the first LSPREAD k blocks: with
+                 * few wavefronts per SIMD a wavefront that issues all of them at once keeps the
+                 * matrix core waiting; spread out, they go between its MFMAs */
+                if (blk < LSPREAD && kt + 1 < nk) dma_tile(kt + 1, cur ^ 1, blk, LSPREAD);
                 if (blk + 1 < BK / KBLK) read_block(cur, (blk + 1) * KBLK, a[(blk + 1) & 1], b[(blk + 1) & 1]);
                 if (blk == BK / KBLK - 1) {
                     __builtin_amdgcn_s_waitcnt(0x0070);      /* vmcnt(0), lgkmcnt(0) */

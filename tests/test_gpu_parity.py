@@ -41,13 +41,14 @@ def key_of(category, name, args):
     return Task(category, name, None, args, "rocm", 0).key
 
 
-def gcfg(M, N, K, wm, rm, wn, rn, mf, bk, sk=1, st=2, gm=4, xcd=1, wk=0, ks=0):
+def gcfg(M, N, K, wm, rm, wn, rn, mf, bk, sk=1, st=2, gm=4, xcd=1, wk=0, ks=0, ls=1):
     """st = pipeline depth; wk=1: the sk K-partitions are wavefront groups of one workgroup;
-    ks > 0: balanced K streaming with ks workgroups per compute unit."""
+    ks > 0: balanced K streaming with ks workgroups per compute unit; ls: k blocks over which
+    depth 8 spreads the loads of the next tile."""
     c = {k: [] for k in KEYS}
     c["spatial"] = [[ceil_div(M, wm * rm * mf), wm, rm, mf], [ceil_div(N, wn * rn * mf), wn, rn, mf]]
     c["reduce"] = [[sk, K // (sk * bk), bk]]
-    c["unroll"], c["fuse"], c["reorder"] = [[st, 1]], [[gm]], [[xcd, wk, ks] if ks else [xcd, wk]]
+    c["unroll"], c["fuse"], c["reorder"] = [[st, ls]], [[gm]], [[xcd, wk, ks] if ks else [xcd, wk]]
     return c
 
 
@@ -295,6 +296,8 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     (128, 288, 128, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=48, st=8), [-1, -1]),            # three k blocks per tile
     (320, 768, 192, dict(wm=2, rm=1, wn=2, rn=2, mf=16, bk=32, st=8, ks=1), [-1, -1]),      # K streaming: segments of any length
     (256, 512, 256, dict(wm=1, rm=2, wn=2, rn=1, mf=16, bk=32, sk=4, wk=1, st=8), [-1, -1]),  # four k-groups in the workgroup
+    (128, 288, 128, dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=48, st=8, ls=2), [-1, -1]),      # the next tile's loads in two parts
+    (200, 512, 136, dict(wm=2, rm=1, wn=1, rn=2, mf=32, bk=64, st=8, ls=7), [-1, 0]),        # in seven parts, more parts than loads, ragged
 ])
 def test_gemm_f32_direct_to_lds(oracle, M, K, N, kn, pad):
     """Pipeline depths 5 to 7: tiles travel global -> LDS without staging registers."""
@@ -381,6 +384,8 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, st=8), [-1, 0]),      # 1x1, N=392
     ((3, 8, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=2, wn=2, rn=2, mf=16, bk=16, st=8, ks=1), [-1, 4]),   # dilation, K tail, K streaming
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=144, st=8, ks=1), [-1, 0]),  # 36 chunks, K streaming
+    ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=144, st=8, ls=6), [-1, 0]),   # loads spread over six k blocks
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=144, st=8, ks=1, ls=4), [-1, 0]),  # the same with K streaming
 ])
 def test_conv2d_direct_to_lds(oracle, args, kn, pad):
     register(conv2d, "conv2d", "t", args, "rocm", 0)

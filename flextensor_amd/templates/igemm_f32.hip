@@ -386,6 +386,15 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #if BV != 1
 #error "conv mode gathers scalars: BV must be 1"
 #endif
+/* Element e of a thread is chunk tid + e * NT of the B tile. When NT is a whole number of
+ * tile rows and that number is a multiple of the k block (the unit inside which the LDS
+ * permutation moves rows), e only moves the element down by BROW_STEP rows: same pixel. */
+#if (NT % BN == 0) && ((NT / BN) % KBLK == 0)
+#define BROW_LINEAR 1
+#define BROW_STEP (NT / BN)
+#else
+#define BROW_LINEAR 0
+#endif
 #else
 /* a batch of independent GEMMs (flextensor/nn/ops.py:1111-1158) reuses the
  * group index: operand b of every matrix starts b*M*K, b*K*N, b*M*N floats in */
@@ -619,20 +628,8 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const int kbase = kz * KSPLIT_LEN + kg * KGROUP_LEN + kt_lo * BK;
 
 #if MODE == 1
-    /* pixel decomposition of each column this thread gathers */
-    int px_off[EB], px_h[EB], px_w[EB];
+    int px_off[EB], px_h[EB], px_w[EB];      /* pixel decomposition of each column this thread gathers */
     bool px_ok[EB];
-#pragma unroll
-    for (int e = 0; e < EB; ++e) {
-        const int n = n0 + b_col[e];
-        px_ok[e] = (n < N) && (tid + e * NT < B_CHUNKS);
-        const int nn = px_ok[e] ? n : 0;
-        const int b = nn / OHW;
-        const int p = nn % OHW;
-        px_h[e] = (p / CQ) * CSTRH - CPADH;
-        px_w[e] = (p % CQ) * CSTRW - CPADW;
-        px_off[e] = b * (CC * CH * CW) + gi * ((CC / CG) * CH * CW);
-    }
 #endif
 
     /* ---- global loads: raw buffer loads with hardware bounds checking --- */
@@ -646,6 +643,94 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const __amdgpu_buffer_rsrc_t rsrc_b =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, B_BYTES, 0x00020000);
     unsigned a_voff[EA], b_voff[EB];
+#if DTL
+    /* The loads are written as instructions, not through the builtin: the
+     * compiler makes every later LDS read wait for a direct-to-LDS load it
+     * knows of (it cannot tell the two buffers apart), which would undo the
+     * overlap. Completion is tracked by hand: vmcnt(0) before the barrier
+     * that ends an iteration. */
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    auto descriptor = [](const float* base, unsigned bytes) {
+        const unsigned long long p = (unsigned long long)base;
+        i32x4 d;                             /* raw buffer: base, stride 0, bytes, untyped dwords */
+        d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+        d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(p >> 32) & 0xffffu));
+        d[2] = (int)bytes;
+        d[3] = 0x00020000;
+        return d;
+    };
+    const i32x4 desc_a = descriptor(A, (unsigned)A_BYTES);
+    const i32x4 desc_b = descriptor(B, (unsigned)B_BYTES);
+    auto dma16 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
+        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
+    };
+    auto dma4 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
+        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
+    };
+    /* part p of np: the loads e of the tile with e mod np == p (A first, then B) */
+    auto dma_tile_a = [&](int kt, int buf, int part = 0, int nparts = 1) {
+        const int k0 = kbase + kt * BK;
+#pragma unroll
+        for (int e = 0; e < EA; ++e) {
+            if (e % nparts != part) continue;
+            unsigned vo = a_voff[e];
+            if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
+            if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))     /* whole wavefronts only */
+                dma16(desc_a, &As[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
+        }
+    };
+    auto dma_b_one = [&](int kt, int buf, int e) {
+        const int k0 = kbase + kt * BK;
+        {
+            if (!((B_CHUNKS % NT == 0) || (e * NT + wv * 64 < B_CHUNKS))) return;
+#if MODE == 2
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
+            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
+#else
+            /* the wavefront's 64 lanes are 64 consecutive columns of one k row */
+            const int q0 = e * NT + wv * 64;
+            const float* dst = &Bs[buf][(q0 / BN) * SB + (q0 % BN)];
+#if MODE == 0 && defined(BSWZ)
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * (N * 4));
+#elif MODE == 0
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma4(desc_b, dst, vo, k0 * (N * 4));
+#elif KHOIST
+            unsigned vo = b_voff[e];
+            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
+            dma4(desc_b, dst, vo, (k0 / (CR * CS)) * (CH * CW * 4));
+#else
+            const int k = k0 + b_row[e];
+            const int c = k / (CR * CS);
+            const int rs = k % (CR * CS);
+            const int ih = px_h[e] + (rs / CS) * CDILH;
+            const int iw = px_w[e] + (rs % CS) * CDILW;
+            bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+            if (KP != K) ok = ok && (k < K);
+            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
+            dma4(desc_b, dst, vo, 0);
+#endif
+#endif
+        }
+    };
+    auto dma_tile_b = [&](int kt, int buf, int part = 0, int nparts = 1) {
+#pragma unroll
+        for (int e = 0; e < EB; ++e)
+            if ((EA + e) % nparts == part) dma_b_one(kt, buf, e);
+    };
+    auto dma_tile = [&](int kt, int buf, int part = 0, int nparts = 1) {
+        dma_tile_a(kt, buf, part, nparts);
+        dma_tile_b(kt, buf, part, nparts);
+    };
+#endif
 #pragma unroll
     for (int e = 0; e < EA; ++e) {
 #if TA
@@ -661,6 +746,25 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         a_voff[e] = ok ? (unsigned)((gi * M + m) * K + a_col[e]) * 4u : OOB;
 #endif
     }
+#if DTL
+    /* tile 0 of A is requested before the index arithmetic of the gathered operand, which
+     * its round trip then covers */
+    dma_tile_a(0, 0);
+#endif
+#if MODE == 1
+    /* pixel decomposition of each column this thread gathers */
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+        const int n = n0 + b_col[e];
+        px_ok[e] = (n < N) && (tid + e * NT < B_CHUNKS);
+        const int nn = px_ok[e] ? n : 0;
+        const int b = nn / OHW;
+        const int p = nn % OHW;
+        px_h[e] = (p / CQ) * CSTRH - CPADH;
+        px_w[e] = (p % CQ) * CSTRW - CPADW;
+        px_off[e] = b * (CC * CH * CW) + gi * ((CC / CG) * CH * CW);
+    }
+#endif
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
         bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
@@ -673,14 +777,30 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         if (N % BN != 0) ok = ok && (n < N);
         b_voff[e] = ok ? (unsigned)((gi * K + b_row[e]) * N + n) * 4u : OOB;
 #elif KHOIST
+#if BROW_LINEAR
+        /* every element of this lane is the same pixel, BROW_STEP rows of the tile further down:
+         * channel and tap follow from those of element 0 without another division */
+        const int cl0 = b_row[0] / (CR * CS), rs0 = b_row[0] % (CR * CS);
+        const int rsx = rs0 + (e * BROW_STEP) % (CR * CS);
+        const int rs = rsx >= CR * CS ? rsx - CR * CS : rsx;
+        const int cl = cl0 + (e * BROW_STEP) / (CR * CS) + (rsx >= CR * CS ? 1 : 0);
+        const int ih = px_h[0] + (rs / CS) * CDILH;
+        const int iw = px_w[0] + (rs % CS) * CDILW;
+        ok = ok && px_ok[0] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
+        b_voff[e] = ok ? (unsigned)(px_off[0] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
+#else
         const int cl = b_row[e] / (CR * CS);
         const int rs = b_row[e] % (CR * CS);
         const int ih = px_h[e] + (rs / CS) * CDILH;
         const int iw = px_w[e] + (rs % CS) * CDILW;
         ok = ok && px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
         b_voff[e] = ok ? (unsigned)(px_off[e] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
+#endif
 #else
         b_voff[e] = OOB;  /* recomputed for every tile */
+#endif
+#if DTL
+        dma_b_one(0, 0, e);       /* tile 0: each load leaves as soon as its address is known */
 #endif
     }
 
@@ -846,91 +966,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         }
     };
 
-#if DTL
-    /* The loads are written as instructions, not through the builtin: the
-     * compiler makes every later LDS read wait for a direct-to-LDS load it
-     * knows of (it cannot tell the two buffers apart), which would undo the
-     * overlap. Completion is tracked by hand: vmcnt(0) before the barrier
-     * that ends an iteration. */
-    const int wv = __builtin_amdgcn_readfirstlane(wave);
-    auto descriptor = [](const float* base, unsigned bytes) {
-        const unsigned long long p = (unsigned long long)base;
-        i32x4 d;                             /* raw buffer: base, stride 0, bytes, untyped dwords */
-        d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
-        d[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(p >> 32) & 0xffffu));
-        d[2] = (int)bytes;
-        d[3] = 0x00020000;
-        return d;
-    };
-    const i32x4 desc_a = descriptor(A, (unsigned)A_BYTES);
-    const i32x4 desc_b = descriptor(B, (unsigned)B_BYTES);
-    auto dma16 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
-        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
-    };
-    auto dma4 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
-        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
-    };
-    /* part p of np: the loads e of the tile with e mod np == p (A first, then B) */
-    auto dma_tile = [&](int kt, int buf, int part = 0, int nparts = 1) {
-        const int k0 = kbase + kt * BK;
-#pragma unroll
-        for (int e = 0; e < EA; ++e) {
-            if (e % nparts != part) continue;
-            unsigned vo = a_voff[e];
-            if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
-            if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))     /* whole wavefronts only */
-                dma16(desc_a, &As[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
-        }
-#pragma unroll
-        for (int e = 0; e < EB; ++e) {
-            if (!((B_CHUNKS % NT == 0) || (e * NT + wv * 64 < B_CHUNKS))) continue;
-            if ((EA + e) % nparts != part) continue;
-#if MODE == 2
-            unsigned vo = b_voff[e];
-            if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
-            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
-#else
-            /* the wavefront's 64 lanes are 64 consecutive columns of one k row */
-            const int q0 = e * NT + wv * 64;
-            const float* dst = &Bs[buf][(q0 / BN) * SB + (q0 % BN)];
-#if MODE == 0 && defined(BSWZ)
-            unsigned vo = b_voff[e];
-            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
-            dma16(desc_b, &Bs[buf][(e * NT + wv * 64) * 4], vo, k0 * (N * 4));
-#elif MODE == 0
-            unsigned vo = b_voff[e];
-            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
-            dma4(desc_b, dst, vo, k0 * (N * 4));
-#elif KHOIST
-            unsigned vo = b_voff[e];
-            if (KP != K) vo = (k0 + b_row[e] < K) ? vo : OOB;
-            dma4(desc_b, dst, vo, (k0 / (CR * CS)) * (CH * CW * 4));
-#else
-            const int k = k0 + b_row[e];
-            const int c = k / (CR * CS);
-            const int rs = k % (CR * CS);
-            const int ih = px_h[e] + (rs / CS) * CDILH;
-            const int iw = px_w[e] + (rs % CS) * CDILW;
-            bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-            if (KP != K) ok = ok && (k < K);
-            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
-            dma4(desc_b, dst, vo, 0);
-#endif
-#endif
-        }
-    };
-#endif
 
     /* ---- main loop ------------------------------------------------------ */
     /* Tile t travels global -> register set t % PD -> LDS buffer -> MFMA.
      * While tile kt is multiplied, tiles kt+1 .. kt+PD are in registers or in
      * flight; tile kt+1 is written to LDS right after the MFMAs of tile kt. */
 #if DTL
-    dma_tile(0, 0);
+    /* tile 0 was requested above, as early as its addresses were known */
     __builtin_amdgcn_s_waitcnt(0x0F70);      /* vmcnt(0): this wavefront's part of tile 0 is in LDS */
 #else
 #pragma unroll

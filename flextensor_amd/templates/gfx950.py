@@ -171,7 +171,7 @@ class GemmView(object):
 
 GEMM_KINDS = ("gemm", "gemm_int8", "conv2d_nchw", "batch_gemm", "col_gemm")
 
-F32_BK = (8, 16, 32, 48, 64, 72, 144)   # 72/144: whole 3x3 windows per LDS tile
+F32_BK = (8, 16, 32, 48, 64, 72, 128, 144)   # 72/144: whole 3x3 windows per LDS tile
 I8_BK = (64, 128, 256)
 
 

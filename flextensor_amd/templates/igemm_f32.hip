@@ -49,6 +49,11 @@
 //                   per lane: 64 consecutive columns of one k row per
 //                   instruction (BN % 64 == 0, rows may be padded) or whole
 //                   unpadded rows (BN < 64)
+//   FPF             with DTL and two buffers: the MFMA operands are read from LDS one k
+//                   block ahead of their use, and the first block of the next tile right
+//                   behind the barrier, which stands before the last k block's MFMAs
+//   LSPREAD         with FPF: the loads of the next tile are issued in LSPREAD parts in
+//                   front of the first LSPREAD k blocks (1: all before the first)
 //   SK_PER          > 0: balanced K streaming. The work is cut into units of
 //                   one LDS tile step (output tile, k-tile); every workgroup
 //                   takes SK_PER consecutive units, so a workgroup may
@@ -66,7 +71,7 @@
 // lane per 4 k-steps), Bs[BK][BN+BPAD] (n contiguous, read as 32-bit loads).
 // With the swizzle, chunk c of row r lives at chunk c ^ swz(r): 16 lanes that
 // read (or write) the same logical chunk of 16 consecutive rows touch 16
-// different groups of four banks.
+// different groups of four banks (the rows may hold any even number of chunks).
 // Within a k-block of 4*KL values, lane group g of an MFMA takes
 // k = 4*g + s at step s for both operands, so the sum over k is unchanged.
 

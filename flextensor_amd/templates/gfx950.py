@@ -798,10 +798,10 @@ def seed_configs(op, limit=24):
             kps = [kp for kp in view.KP_options if kp % bk == 0]
             if not kps:
                 continue
-            for depth in depths:
-                for stream in streams:
-                    if stream and (i8 or tiles >= 2 * NUM_CUS):
-                        continue
+            # K streaming first where the tiles alone cannot fill the compute units
+            order = [(d, st) for st in (streams[::-1] if tiles < NUM_CUS else streams) for d in depths]
+            for depth, stream in order:
+                if not (stream and (i8 or tiles >= 2 * NUM_CUS)):
                     cfg = _empty_config()
                     cfg["spatial"] = [tm, tn]
                     cfg["reduce"] = [[1, kps[0] // bk, bk]]
@@ -809,7 +809,7 @@ def seed_configs(op, limit=24):
                     cfg["fuse"] = [[8]]
                     cfg["reorder"] = [[1, 0, stream]]
                     out.append(cfg)
-                if not i8 and depth == depths[0] and tiles * 2 <= NUM_CUS:
+                if not i8 and depth == depths[0] and stream == 0 and tiles * 2 <= NUM_CUS:
                     # few tiles and a long K (weights streamed past a small image): K parts across
                     # workgroups, as many as fill the compute units
                     split = 1
@@ -848,7 +848,9 @@ def seed_configs(op, limit=24):
             gi = k % len(groups)
             g = groups[gi]
             if taken[gi] < len(g):
-                picked.append(g[(taken[gi] + gi) % len(g)])
+                # the start moves through the depths with the group; the streaming choice listed
+                # first for the group stays first
+                picked.append(g[(taken[gi] + gi % len(depths)) % len(g)])
                 taken[gi] += 1
             k += 1
         return picked

@@ -1032,6 +1032,22 @@ def test_registered_tasks_default_config_passes_the_gate(key):
     assert 0 < ms < 1e3
 
 
+def _shipped_keys():
+    from flextensor_amd.tuned import load
+    return sorted(load())
+
+
+@pytest.mark.parametrize("key", _shipped_keys())
+def test_every_shipped_entry_passes_the_gate(key):
+    """Each line of the shipped log of tuned points lowers with today's
+    templates and its kernels match the default-schedule kernels on the
+    device (fp32 within 1e-5 of the largest value, int32 identical)."""
+    s, bufs = schedule_with_config(key, tuned_configs(key))
+    s.compile()
+    ms = Measurer(key).evaluate(s, number=3, warmup=1, warm_ms=0)
+    assert 0 < ms < 1e3
+
+
 def test_correctness_gate_rejects_wrong_output():
     key = "gemm_gemm_(256, 256, 256)_rocm(0)"
     m = Measurer(key)

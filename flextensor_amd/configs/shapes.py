@@ -109,6 +109,9 @@ depthwise_shapes = [
     (1, 96, 14, 14, 6, 3, 3, 2, 1, 1),
     (1, 160, 7, 7, 6, 3, 3, 1, 1, 1),
 ]
+# the same layers at batch 8 and 16 (flextensor/configs/depthwise_config.py:12-31)
+depthwise_shapes_b8 = [(8,) + s[1:] for s in depthwise_shapes]
+depthwise_shapes_b16 = [(16,) + s[1:] for s in depthwise_shapes]
 
 # 1x1 convolution 1024 -> 512 on 14x14 with 4..32 groups
 grouped_shapes = [(1, 1024, 14, 14, 512, 1, 1, 1, 0, 1, g) for g in (4, 8, 16, 32)]

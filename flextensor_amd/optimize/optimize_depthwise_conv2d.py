@@ -5,11 +5,13 @@ flextensor/optimize/optimize_depthwise_conv2d.py:18-120 for the gfx950 backend.
 """
 import argparse
 
-from ..configs.shapes import baseline_depthwise_shapes, depthwise_shapes
+from ..configs.shapes import (baseline_depthwise_shapes, depthwise_shapes, depthwise_shapes_b8,
+                              depthwise_shapes_b16)
 from ..task import Task
 from .common import init_arg_parser, run_driver
 
-SHAPES = {"baseline": baseline_depthwise_shapes, "mobile": depthwise_shapes}
+SHAPES = {"baseline": baseline_depthwise_shapes, "mobile": depthwise_shapes,
+          "mobile_b8": depthwise_shapes_b8, "mobile_b16": depthwise_shapes_b16}
 
 
 def make_task(index, shape, args):

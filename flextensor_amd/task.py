@@ -12,10 +12,10 @@ from .nn import conv2d_nchw, depthwise_conv2d_nchw, gemm as op_gemm, gemm_int8 a
 from .space import EnumSpace
 from .te import placeholder
 from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8, grouped_shapes, dilation_shapes,
-                             depthwise_shapes, baseline_conv_shapes, baseline_depthwise_shapes,
-                             baseline_gemm_shapes, baseline_gemm_int8_shapes, google_shapes, res_shapes,
-                             squeeze_shapes, vgg_16_shapes, test_conv_shapes, mobilev2_shapes,
-                             overfeat_shapes)
+                             depthwise_shapes, depthwise_shapes_b8, depthwise_shapes_b16,
+                             baseline_conv_shapes, baseline_depthwise_shapes, baseline_gemm_shapes,
+                             baseline_gemm_int8_shapes, google_shapes, res_shapes, squeeze_shapes,
+                             vgg_16_shapes, test_conv_shapes, mobilev2_shapes, overfeat_shapes)
 
 # table name -> conv2d shapes, the names of flextensor/task.py:274-284 plus this backend's benchmark shapes
 conv2d_shape_dict = {
@@ -156,7 +156,8 @@ def _register_all():
                 batch, in_c, h, w, out_c, k, _, stride, pad, dil, groups = shape
                 register(conv2d, "conv2d", name, (batch, in_c, h, w, out_c, k, stride, pad, dil, groups),
                          ROCM_TARGET, j)
-        for shape in depthwise_shapes + baseline_depthwise_shapes:
+        for shape in depthwise_shapes + depthwise_shapes_b8 + depthwise_shapes_b16 + \
+                baseline_depthwise_shapes:
             batch, in_c, h, w, factor, k_h, k_w, stride, pad, dil = shape
             register(depthwise_conv2d, "conv2d", "depthwise",
                      (batch, in_c, h, w, factor, k_h, stride, pad, dil), ROCM_TARGET, j)

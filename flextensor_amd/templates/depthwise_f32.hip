@@ -15,7 +15,9 @@
 // halo left and right of a lane's four columns comes from the neighbouring
 // lanes through DPP wavefront shifts instead of two more global loads; each
 // wavefront then uses a multiple of TILES_W lanes so that neighbours along W
-// are always in the same wavefront).
+// are always in the same wavefront), MFUSE (1: with FACT > 1 kernels per input
+// channel a lane loads its input patch once and computes the patch of all
+// FACT output planes from it, instead of one lane per output plane).
 // LDSP > 0 selects the plane-staged variant instead: a workgroup streams LDSP
 // whole planes into LDS with 128-bit loads in pure copy order (every input
 // element is fetched once, no halo re-reads), computes from LDS, where a zero
@@ -59,6 +61,11 @@
 #else
 #define WX 0
 #endif
+#ifdef FT_MFUSE
+#define MFUSE FT_MFUSE    /* a lane computes all FACT output planes of its input patch */
+#else
+#define MFUSE 0
+#endif
 #define CB FT_CB
 #define CC FT_CC
 #define CH FT_CH
@@ -79,26 +86,31 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 #define PLANES (CB * CC * FACT)
+#define FM (MFUSE ? FACT : 1)            /* output planes per lane patch */
 #define TILES_H ((CP + TH - 1) / TH)
 #define TILES_W ((CQ + TW - 1) / TW)
-#define ITEMS (PLANES * TILES_H * TILES_W)
+#define ITEMS (PLANES / FM * TILES_H * TILES_W)
 #define IH_T ((TH - 1) * STRH + (CR - 1) * DILH + 1)
 #define IW_T ((TW - 1) * STRW + (CS - 1) * DILW + 1)
 
-/* 128-bit path: same-size stride-1 convolution whose rows keep 16-byte
- * alignment; the four centre columns of a patch come in as one vector. */
-#if (TW == 4) && (STRW == 1) && (CW % 4 == 0) && (CQ == CW) && (PADW + 4 <= IW_T)
+/* 128-bit path: a convolution with stride 1 or 2 along W whose output rows
+ * are 1/STRW of the input rows and whose rows keep 16-byte alignment; the
+ * 4 * STRW input columns from the patch's first output column on come in as
+ * STRW vectors (of a ragged last patch they may run into the next row: those
+ * elements only feed outputs that are not stored). */
+#if (TW == 4) && (STRW <= 2) && (CW % 4 == 0) && (CQ * STRW == CW) && (PADW + 4 * STRW <= IW_T)
 #define VEC_IN 1
 #else
 #define VEC_IN 0
 #endif
+#define NVEC STRW
 #if (TW == 4) && (CQ % 4 == 0)
 #define VEC_OUT 1
 #else
 #define VEC_OUT 0
 #endif
 #if SHFL
-#if !(VEC_IN && CS == 3 && DILW == 1 && PADW == 1 && TILES_W <= 64)
+#if !(VEC_IN && STRW == 1 && CS == 3 && DILW == 1 && PADW == 1 && TILES_W <= 64)
 #error "SHFL needs the 128-bit input path with a 3-wide kernel, dilation 1, padding 1"
 #endif
 #define LPW ((64 / TILES_W) * TILES_W)   /* lanes of a wavefront that carry work */
@@ -316,9 +328,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
      * wavefronts move the same bytes. */
     bool live[IPL];
     int tw[IPL], ovo[IPL], oh0[IPL];
-    float wreg[IPL][CR][CS];
+    float wreg[IPL][FM][CR][CS];
 #if (SHFL || VEC_IN)
-    f32x4 rows[IPL][IH_T];
+    f32x4 rows[IPL][IH_T][NVEC];
 #if !SHFL
     float halo[IPL][IH_T][IW_T];
 #endif
@@ -340,18 +352,25 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         tw[k] = gid % TILES_W;
         const int th = (gid / TILES_W) % TILES_H;
         const int plane = gid / (TILES_W * TILES_H);
+#if MFUSE
+        /* plane counts input planes; its output planes are plane * FACT .. plane * FACT + FACT - 1 */
+        const int co = (plane % CC) * FACT;
+        const int xplane = plane * (CH * CW);
+#else
         const int b = plane / (CC * FACT);
         const int co = plane % (CC * FACT);
         const int ci = co / FACT;
         const int xplane = (b * CC + ci) * (CH * CW);      /* first element of the input plane */
+#endif
         oh0[k] = th * TH;
         const int ow0 = tw[k] * TW;
         const int ih0 = oh0[k] * STRH - PADH;
         const int iw0 = ow0 * STRW - PADW;
-        ovo[k] = plane * (CP * CQ) + oh0[k] * CQ + ow0;     /* first output element of the patch */
-        {
+        ovo[k] = plane * FM * (CP * CQ) + oh0[k] * CQ + ow0;     /* first output element of the patch */
+#pragma unroll
+        for (int m = 0; m < FM; ++m) {
             /* the kernel's CR*CS taps: 128-bit loads (dword-aligned is enough for buffer loads) and a tail */
-            const unsigned wo = live[k] ? (unsigned)(co * (CR * CS)) * 4u : OOB;
+            const unsigned wo = live[k] ? (unsigned)((co + m) * (CR * CS)) * 4u : OOB;
             float wflat[(CR * CS + 3) / 4 * 4];
 #pragma unroll
             for (int t = 0; t + 4 <= CR * CS; t += 4) {
@@ -365,7 +384,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
             for (int r = 0; r < CR; ++r)
 #pragma unroll
                 for (int s = 0; s < CS; ++s)
-                    wreg[k][r][s] = wflat[r * CS + s];
+                    wreg[k][m][r][s] = wflat[r * CS + s];
         }
         /* one element of input row ih (any int), column iw (any int); zero outside the image */
         auto load1 = [&](int ih, int iw) -> float {
@@ -376,19 +395,21 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #if (SHFL || VEC_IN)
 #pragma unroll
         for (int y = 0; y < IH_T; ++y) {
-            /* the four centre columns of input row ih0 + y */
+            /* the 4 * STRW centre columns of input row ih0 + y */
             const int ih = ih0 + y;
             const bool row_ok = live[k] && (unsigned)ih < (unsigned)CH;
-            const unsigned vo = row_ok ? (unsigned)(xplane + ih * CW + ow0) * 4u : OOB;
-            rows[k][y] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo, 0, LD_AUX));
+            const unsigned vo = row_ok ? (unsigned)(xplane + ih * CW + ow0 * STRW) * 4u : OOB;
+#pragma unroll
+            for (int v = 0; v < NVEC; ++v)
+                rows[k][y][v] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, (int)vo, v * 16, LD_AUX));
         }
 #if !SHFL
-        /* the halo columns left and right of the centre vector */
+        /* the halo columns left and right of the centre vectors */
 #pragma unroll
         for (int y = 0; y < IH_T; ++y)
 #pragma unroll
             for (int j = 0; j < IW_T; ++j)
-                if (j < PADW || j >= PADW + 4) halo[k][y][j] = load1(ih0 + y, iw0 + j);
+                if (j < PADW || j >= PADW + 4 * NVEC) halo[k][y][j] = load1(ih0 + y, iw0 + j);
 #endif
 #else
 #pragma unroll
@@ -399,7 +420,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     }
 
 #pragma unroll
-    for (int k = 0; k < IPL; ++k) {
+    for (int k = 0; k < IPL; ++k)
+#pragma unroll
+    for (int m = 0; m < FM; ++m) {
         float acc[TH][TW];
 #pragma unroll
         for (int i = 0; i < TH; ++i)
@@ -411,7 +434,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
             float in[IW_T];
 #if SHFL
             {
-                const f32x4 v = rows[k][y];
+                const f32x4 v = rows[k][y][0];
                 /* column ow0-1 is the last column of the lane below, column ow0+4
                  * the first column of the lane above; image borders read zero */
                 const float v0 = v[0], v3 = v[3];
@@ -423,10 +446,10 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
             }
 #elif VEC_IN
             {
-                const f32x4 v = rows[k][y];
 #pragma unroll
                 for (int j = 0; j < IW_T; ++j)
-                    in[j] = (j >= PADW && j < PADW + 4) ? v[(j - PADW) & 3] : halo[k][y][j];
+                    in[j] = (j >= PADW && j < PADW + 4 * NVEC) ? rows[k][y][((j - PADW) >> 2) % NVEC][(j - PADW) & 3]
+                                                               : halo[k][y][j];
             }
 #else
 #pragma unroll
@@ -442,7 +465,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                         for (int j = 0; j < TW; ++j)
 #pragma unroll
                             for (int s = 0; s < CS; ++s)
-                                acc[i][j] += in[j * STRW + s * DILW] * wreg[k][r][s];
+                                acc[i][j] += in[j * STRW + s * DILW] * wreg[k][m][r][s];
                     }
                 }
             }
@@ -455,13 +478,13 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #if VEC_OUT
             f32x4 v;
             v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];
-            const unsigned vo = row_ok ? (unsigned)(ovo[k] + i * CQ) * 4u : OOB;
+            const unsigned vo = row_ok ? (unsigned)(ovo[k] + m * (CP * CQ) + i * CQ) * 4u : OOB;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ro, (int)vo, 0, ST_AUX);
 #else
 #pragma unroll
             for (int j = 0; j < TW; ++j) {
                 const bool ok = row_ok && (CQ % TW == 0 || tw[k] * TW + j < CQ);
-                const unsigned vo = ok ? (unsigned)(ovo[k] + i * CQ + j) * 4u : OOB;
+                const unsigned vo = ok ? (unsigned)(ovo[k] + m * (CP * CQ) + i * CQ + j) * 4u : OOB;
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, acc[i][j]), ro, (int)vo, 0, ST_AUX);
             }
 #endif

@@ -246,6 +246,8 @@ SPECIAL_DEFAULTS = {
     "lds_planes": [0],
     "lane_items": [1],
     "row_exchange": [0],
+    # depthwise with several kernels per input channel: 1 = a lane computes its patch for all of them
+    "kernel_fuse": [1],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -268,7 +270,8 @@ def special_knobs(kind):
         return {"lds_pad": [[-1, 0], [4, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]],
-                "lane_items": [[1], [2], [3], [4], [6], [8]], "row_exchange": [[0], [1], [2], [3], [4]]}
+                "lane_items": [[1], [2], [3], [4], [6], [8]], "row_exchange": [[0], [1], [2], [3], [4]],
+                "kernel_fuse": [[1], [0]]}
     return {}
 
 
@@ -539,17 +542,19 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     ih_t = (th - 1) * st_h + (r_ext - 1) * dl_h + 1
     iw_t = (tw - 1) * st_w + (s_ext - 1) * dl_w + 1
     # the 128-bit input path requests every row of the patch before the first is used
-    vec_rows = (tw == 4 and st_w == 1 and w % 4 == 0 and q == w and pad_w + 4 <= iw_t)
+    vec_rows = (tw == 4 and st_w <= 2 and w % 4 == 0 and q * st_w == w and pad_w + 4 * st_w <= iw_t)
+    # kernel_fuse: with several kernels per input channel a lane computes its patch for all of them
+    fm = a["factor"] if int(_special(special, "kernel_fuse")[0]) else 1
     # lane_items: patches per lane, all requested before the first is computed
     ipl = int(_special(special, "lane_items")[0])
     if ipl < 1 or ipl > 16:
         raise InvalidConfig("lane_items is 1 .. 16")
-    if th * tw + ipl * ((ih_t * iw_t if vec_rows else ih_t * iw_t) + r_ext * s_ext) > 220:
+    if th * tw + ipl * (ih_t * iw_t + fm * r_ext * s_ext) > 220:
         raise InvalidConfig("lane patches need too many registers")
     if max(b * c * h * w, b * cout * p * q) * 4 >= 2 ** 31:
         raise InvalidConfig("tensors of 2 GiB or more are not addressable by the buffer accesses")
     nt = waves * 64
-    items = b * cout * ceil_div(p, th) * ceil_div(q, tw)
+    items = b * (cout // fm) * ceil_div(p, th) * ceil_div(q, tw)
     ldsp = int(_special(special, "lds_planes")[0])
     nt_mode = int(_special(special, "nt_store")[0])     # bit 0: non-temporal stores, bit 1: non-temporal loads
     steps = dict(STRH=st_h, STRW=st_w, PADH=pad_h, PADW=pad_w, DILH=dl_h, DILW=dl_w)
@@ -592,7 +597,7 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     shfl = int(_special(special, "halo_shfl")[0])
     tiles_w = ceil_div(q, tw)
     if shfl:
-        if not (vec_rows and s_ext == 3 and dl_w == 1 and pad_w == 1 and tiles_w <= 64):
+        if not (vec_rows and st_w == 1 and s_ext == 3 and dl_w == 1 and pad_w == 1 and tiles_w <= 64):
             raise InvalidConfig("the shuffled halo needs the 128-bit input path of a 3-wide pad-1 layer")
         lanes = (64 // tiles_w) * tiles_w
         grid_x = ceil_div(ceil_div(items, lanes), waves * ipl)
@@ -602,6 +607,8 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
              CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=a["factor"], CP=p, CQ=q, **steps)
     if ipl > 1:
         D.update(IPL=ipl)
+    if fm > 1:
+        D.update(MFUSE=1)
     return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
                        (nt, 1, 1),
                        [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]

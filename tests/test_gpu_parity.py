@@ -809,6 +809,39 @@ def test_depthwise_vs_oracle(oracle, args, th, tw, waves):
     assert rel(out, ref) <= TOL
 
 
+@pytest.mark.parametrize("args,th,tw,waves", [
+    ((2, 6, 16, 32, 6, 3, 2, 1, 1), 2, 4, 2),     # stride 2, rows of whole vectors: two 128-bit loads per patch row
+    ((1, 5, 14, 28, 6, 3, 2, 1, 1), 1, 4, 1),     # 14 output columns: the last patch of a row is ragged
+    ((1, 4, 14, 14, 6, 3, 1, 1, 1), 2, 4, 1),     # stride 1, rows that are no multiple of four floats (scalar loads)
+    ((2, 3, 12, 16, 3, 3, 1, 1, 1), 3, 4, 2),     # stride 1, one 128-bit load per patch row, factor 3
+    ((1, 4, 16, 16, 2, 3, 2, 2, 2), 2, 4, 1),     # stride 2, dilation 2, padding 2: two halo columns on the left
+    ((1, 4, 13, 16, 2, 3, 2, 1, 2), 2, 4, 1),     # stride 2, dilation 2, padding 1: output rows are not half rows
+    ((1, 3, 9, 11, 4, 3, 2, 1, 1), 2, 2, 1),      # odd plane, two outputs per lane row
+])
+def test_depthwise_kernels_of_a_channel_fused_vs_oracle(oracle, args, th, tw, waves):
+    """Several kernels per input channel: a lane loads its input patch once and
+    computes the patch of every output plane of the channel (kernel_fuse 1),
+    or lanes own single output planes (0); stride 2 reads two vectors per row."""
+    register(depthwise_conv2d, "conv2d", "depthwise", args, "rocm", 0)
+    key = key_of("conv2d", "depthwise", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
+    b_, co, p, q = ref.shape
+    for fuse in (1, 0):
+        for items in (1, 2):
+            cfgs = conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves),
+                             special=[[0], [0], [0], [items], [0], [fuse]])
+            s, _ = schedule_with_config(key, cfgs)
+            assert s.specs[-1].defines.get("MFUSE", 0) == fuse
+            out = run_plan(key, cfgs, [x, w])
+            assert rel(out, ref) <= TOL, (fuse, items)
+    # borders: a constant image must give border sums with missing taps
+    ones = np.ones_like(x)
+    out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves)), [ones, w])
+    assert rel(out, oracle.depthwise_nchw_np(ones, w, args[6], args[7], args[8])) <= TOL
+
+
 @pytest.mark.parametrize("args,th,waves", [
     ((2, 16, 28, 28, 1, 3, 1, 1, 1), 7, 4),       # 7 lanes per row, 63 lanes per wavefront
     ((1, 5, 8, 12, 1, 3, 1, 1, 1), 4, 1),         # 3 lanes per row, last wavefront partly idle

@@ -70,12 +70,23 @@ def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, grou
     padded = zero_pad2d(inputs, padding=padding)
     out_shape = (batch, out_c, out_h, out_w)
     axis = [IterVar(n, e) for n, e in zip("bchw", out_shape)]
-    raxis = [IterVar("rc", c_per_group, "reduce"), IterVar("rw", k_w, "reduce"),
-             IterVar("rh", k_h, "reduce")]
-    op = ComputeOp("compute", "conv2d_nchw", out_shape, inputs.dtype, axis, raxis,
-                   [padded, weight],
-                   {"stride": stride, "padding": padding, "dilation": dilation,
-                    "groups": int(groups), "in_shape": inputs.shape})
+    if c_per_group == 1 and groups > 1:
+        # one input channel per group (MobileNet's stages in flextensor/configs/conv2d_config.py:58-78):
+        # rc has a single value, output channel k reads input channel k // (out_c / groups) and the
+        # weight [out_c, 1, kh, kw] is the depthwise weight [C, factor, kh, kw] in memory, so this is
+        # the depthwise operator (ops.py:622-678), with the same reduce order rw, rh, and takes its kernel
+        raxis = [IterVar("rw", k_w, "reduce"), IterVar("rh", k_h, "reduce")]
+        op = ComputeOp("compute", "depthwise_conv2d_nchw", out_shape, inputs.dtype, axis, raxis,
+                       [padded, weight],
+                       {"stride": stride, "padding": padding, "dilation": dilation,
+                        "factor": out_c // groups, "in_shape": inputs.shape})
+    else:
+        raxis = [IterVar("rc", c_per_group, "reduce"), IterVar("rw", k_w, "reduce"),
+                 IterVar("rh", k_h, "reduce")]
+        op = ComputeOp("compute", "conv2d_nchw", out_shape, inputs.dtype, axis, raxis,
+                       [padded, weight],
+                       {"stride": stride, "padding": padding, "dilation": dilation,
+                        "groups": int(groups), "in_shape": inputs.shape})
     if bias is not None:
         return bias_add_nchw(op.output(0), bias)
     return op.output(0)

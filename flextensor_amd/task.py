@@ -123,6 +123,8 @@ def _attach_default_knobs(task):
             gemm_conv2d: "col_gemm", depthwise_conv2d: "depthwise_conv2d_nchw"}.get(task.func)
     if kind is None:
         return
+    if kind == "conv2d_nchw" and len(task.args) > 9 and task.args[9] > 1 and task.args[1] == task.args[9]:
+        kind = "depthwise_conv2d_nchw"        # one input channel per group: nn.conv2d_nchw builds that operator
     for key, knobs in special_knobs(kind).items():
         if key not in task.special_space:
             task.set_specific_space(key, "enum", knobs)

@@ -41,6 +41,8 @@ def _from_direct_convolution(key, table):
     if direct is None or len(direct.op_config_lst) != 2:
         return None
     pad_cfg, conv_cfg = direct.op_config_lst
+    if len(conv_cfg.get("spatial") or []) != 2:
+        return None      # one channel per group: the direct task is tuned for the depthwise kernel
     empty = {k: [] for k in conv_cfg}
     graph = dict(direct.graph_config or {})
     pad_inline = (graph.get("inline") or [[1, 0]])[0][0]

@@ -699,7 +699,7 @@ CONV_CASES = [
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=16, bk=16, sk=3, wk=1, st=3)),
     ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=32, sk=2, wk=1, st=4)),
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72)),              # groups 4, whole windows
-    ((2, 24, 10, 10, 24, 3, 1, 1, 1, 24), dict(wm=1, rm=1, wn=1, rn=2, mf=16, bk=16)),             # groups = channels
+    ((2, 24, 10, 10, 24, 3, 1, 1, 1, 12), dict(wm=1, rm=1, wn=1, rn=2, mf=16, bk=16)),             # two channels per group, K=18 -> 32
     ((1, 16, 14, 14, 32, 3, 2, 1, 1, 2), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=8, sk=3)),         # groups 2, split-K atomics
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, ks=1)),        # groups 4, K streaming
     ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16, ks=1, st=3)),   # K streaming, padded K
@@ -727,6 +727,34 @@ def test_conv2d_vs_oracle(oracle, args, kn):
         out = run_plan(key, conv_cfgs(cfg, inline), [x, w])
         assert rel(out, ref) <= TOL, inline
         assert rel(out, oracle.conv2d_nchw_np(x, w, st, pd, dl, g)) <= TOL
+
+
+@pytest.mark.parametrize("args", [
+    (2, 24, 10, 10, 24, 3, 1, 1, 1, 24),          # groups = channels, one kernel per channel
+    (1, 8, 12, 16, 48, 3, 2, 1, 1, 8),            # six kernels per channel, stride 2 (a MobileNet stage)
+    (2, 5, 9, 11, 10, 3, 1, 1, 2, 5),             # two kernels per channel, dilation 2
+])
+def test_conv2d_with_one_channel_per_group_takes_the_depthwise_kernel(oracle, args):
+    """conv2d_nchw with groups = input channels is the depthwise operator (weight
+    [K, 1, kh, kw] = [C, K/C, kh, kw] in memory): the plan holds the depthwise
+    kernel and its result is the grouped convolution's."""
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    key = key_of("conv2d", "t", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    assert ops[0].kind == "depthwise_conv2d_nchw" and ops[0].attrs["factor"] == args[4] // args[1]
+    assert "row_exchange" in TASK_TABLE[key].special_space
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
+    assert ref.shape == bufs[-1].shape
+    b_, co, p, q = ref.shape
+    s, _ = schedule_with_config(key, Config([], None))
+    assert [sp.kernel for sp in s.specs] == ["depthwise_f32"]
+    assert rel(run_plan(key, Config([], None), [x, w]), ref) <= TOL
+    for inline in ([1, 0], [0, 0]):
+        for fuse in (1, 0):
+            cfgs = conv_cfgs(dcfg(b_, co, p, q, min(2, p), min(4, q), 2), inline, special=[[0], [0], [0], [1], [0], [fuse]])
+            assert rel(run_plan(key, cfgs, [x, w]), ref) <= TOL, (inline, fuse)
 
 
 def test_conv2d_and_depthwise_with_row_column_pairs(oracle):

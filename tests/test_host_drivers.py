@@ -114,6 +114,11 @@ def test_tuned_convolution_points_carry_over_to_the_im2col_form():
     d, _ = schedule_with_config(direct, lookup(direct))
     assert [k.defines for k in s.specs] == [k.defines for k in d.specs] and not s.intermediates
     assert lookup("gemm_conv2d_nothing_(1,)_rocm(0)") is None
+    # one input channel per group: the direct task is the depthwise operator, tuned for another kernel
+    mobile = "conv2d_mobile_v21_(1, 16, 112, 112, 96, 3, 2, 1, 1, 16)_rocm(0)"
+    assert mobile in load() and lookup("gemm_" + mobile) is None
+    s, _ = schedule_with_config(mobile, lookup(mobile))
+    assert [k.kernel for k in s.specs] == ["depthwise_f32"] and s.specs[0].defines["MFUSE"] == 1
 
 
 def test_layer_tuned_at_another_batch_size_seeds_the_search():

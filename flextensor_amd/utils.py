@@ -5,7 +5,6 @@ get_factor_lst :82-93, any_factor_split :106-128, gen_enum :218-221,
 gen_group :235-242, is_power_of_x :257-259, test_allclose :267-277).
 The Android/RPC helper (RpcInfo) is accepted for call compatibility only.
 """
-import math
 from collections import namedtuple
 
 import numpy as np

@@ -5,7 +5,6 @@ K streaming sums in a fixed order, so the two paths must agree bit for bit."""
 import ctypes
 import os
 
-import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -17,7 +16,7 @@ if not torch.cuda.is_available() and os.environ.get("FT_TESTS_COMPILE_ONLY") != 
 from flextensor_amd import runtime as rt  # noqa: E402
 from flextensor_amd.measure import seeded_inputs  # noqa: E402
 from flextensor_amd.scheduler import schedule_with_config  # noqa: E402
-from flextensor_amd.task import TASK_TABLE, Task, register, conv2d  # noqa: E402
+from flextensor_amd.task import Task, register, conv2d  # noqa: E402
 from flextensor_amd.utils import Config, ceil_div  # noqa: E402
 
 KEYS = ["fuse", "spatial", "reduce", "reorder", "inline", "unroll", "merge", "special"]

@@ -162,10 +162,18 @@ class GemmView(object):
         if self.dtype == "int8":
             self.KP_options = [ceil_div(self.K, 64) * 64]
         else:
-            self.KP_options = [ceil_div(self.K, 16) * 16]
+            self.KP = ceil_div(self.K, 16) * 16
+            self.KP_options = [self.KP]
             if self.K % 8 == 0 and self.K % 16 != 0:
                 # e.g. K = 72: unpadded for 32x32x2 tiles of 8 or 72, padded to 80 for 16x16x4
                 self.KP_options.insert(0, self.K)
+            if not any(kp % 32 == 0 or kp % 48 == 0 or kp % 72 == 0 for kp in self.KP_options):
+                # an awkward K (400 = 16 channels x 5x5) only divides into LDS tiles of 8 or 16: every
+                # tile is a round trip to memory, 25 in a row. Up to an eighth of zero padding (the load
+                # predicates supply it) buys tiles of 32 .. 144: 416, 432, 448 for K = 400
+                wider = {ceil_div(self.K, bk) * bk for bk in (32, 48, 64, 72, 144)}
+                self.KP_options += sorted(kp for kp in wider if kp > self.KP and kp * 8 <= self.K * 9)
+            return
         self.KP = self.KP_options[-1]
 
 

@@ -700,6 +700,11 @@ CONV_CASES = [
     ((1, 64, 28, 28, 64, 3, 1, 1, 1, 1), dict(wm=4, rm=1, wn=1, rn=1, mf=16, bk=32, sk=2, wk=1, st=4)),
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72)),              # groups 4, whole windows
     ((2, 24, 10, 10, 24, 3, 1, 1, 1, 12), dict(wm=1, rm=1, wn=1, rn=2, mf=16, bk=16)),             # two channels per group, K=18 -> 32
+    # K = 400 has no LDS tile wider than 16: zero-padded to 448 = 7 x 64 and 432 = 3 x 144 (the last tile holds 16 real columns)
+    ((2, 16, 14, 14, 48, 5, 1, 2, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=64, st=3, kp=448)),
+    ((2, 16, 14, 14, 48, 5, 1, 2, 1, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=144, st=5, kp=432)),
+    ((2, 16, 14, 14, 48, 5, 1, 2, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=144, st=8, ls=4, kp=432)),
+    ((2, 16, 14, 14, 48, 5, 1, 2, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=32, st=2, kp=416, wk=1, sk=13)),
     ((1, 16, 14, 14, 32, 3, 2, 1, 1, 2), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=8, sk=3)),         # groups 2, split-K atomics
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=72, ks=1)),        # groups 4, K streaming
     ((1, 8, 17, 13, 24, 3, 2, 1, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16, ks=1, st=3)),   # K streaming, padded K
@@ -721,7 +726,8 @@ def test_conv2d_vs_oracle(oracle, args, kn):
     ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
     assert ref.shape == bufs[-1].shape
     M, N, K = ko // g, nb * ref.shape[2] * ref.shape[3], (c // g) * ks * ks
-    kp = K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16
+    kn = dict(kn)
+    kp = kn.pop("kp", K if K % kn["bk"] == 0 else ceil_div(K, 16) * 16)
     cfg = gcfg(M, N, kp, **kn)
     for inline in ([1, 0], [0, 0]):
         out = run_plan(key, conv_cfgs(cfg, inline), [x, w])

@@ -95,10 +95,9 @@ def conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1, grou
 def depthwise_conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilation=1):
     """O[b,c,h,w] = sum_{rw,rh} P[b, c//f, h*s+rh*d, w*s+rw*d] * W[c//f, c%f, rh, rw].
 
-    Follows flextensor/nn/ops.py:622-678; weight layout [C, factor, kh, kw].
+    Follows flextensor/nn/ops.py:622-678; weight layout [C, factor, kh, kw];
+    a bias (one entry per output channel) is its own stage behind it (ops.py:673-677).
     """
-    if bias is not None:
-        raise NotImplementedError("bias epilogue is not part of the tuned path")
     batch, in_c, in_h, in_w = inputs.shape
     w_c, factor, k_h, k_w = weight.shape
     if w_c != in_c:
@@ -116,6 +115,8 @@ def depthwise_conv2d_nchw(inputs, weight, bias=None, stride=1, padding=0, dilati
                    [padded, weight],
                    {"stride": stride, "padding": padding, "dilation": dilation,
                     "factor": int(factor), "in_shape": inputs.shape})
+    if bias is not None:
+        return bias_add_nchw(op.output(0), bias)
     return op.output(0)
 
 

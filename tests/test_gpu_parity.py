@@ -446,6 +446,51 @@ def test_conv2d_with_bias(oracle, args, kn, pad):
     assert rel(out.cpu().numpy(), ref) <= TOL
 
 
+def _depthwise_bias(N, C, H, W, factor, k, stride=1, padding=0, dilation=1):
+    from flextensor_amd.nn import depthwise_conv2d_nchw
+    Img = placeholder((N, C, H, W), name="Img")
+    Wt = placeholder((C, factor, k, k), name="W")
+    bias = placeholder((C * factor,), name="bias")
+    Out = depthwise_conv2d_nchw(Img, Wt, bias, stride=stride, padding=padding, dilation=dilation)
+    return [Out.op], [Img, Wt, bias, Out]
+
+
+def test_depthwise_and_one_channel_groups_with_bias(oracle):
+    """[Padding, depthwise, bias] (flextensor/nn/ops.py:673-677): the bias runs as its own kernel
+    behind the depthwise kernel; conv2d_nchw with groups = channels and a bias builds the same graph."""
+    for args in ((2, 6, 12, 16, 1, 3, 1, 1, 1), (1, 4, 14, 16, 6, 3, 2, 1, 1)):
+        register(_depthwise_bias, "conv2d", "dw_bias", args, "rocm", 0)
+        key = key_of("conv2d", "dw_bias", args)
+        ops, bufs = TASK_TABLE[key].func(*args)
+        x, w, bias = seeded_inputs(bufs, seed=sum(args))
+        ref = oracle.bias_add_nchw_np(oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8]), bias)
+        b_, co, p, q = ref.shape
+        s, _ = schedule_with_config(key, Config([], None))
+        assert [k.kernel for k in s.specs] == ["depthwise_f32", "bias_add_nchw_f32"]
+        assert rel(run_plan(key, Config([], None), [x, w, bias]), ref) <= TOL
+        gc = {k: [] for k in KEYS}
+        gc["inline"], gc["merge"] = [[1, 0, 0]], [[0, 0, 0]]
+        configs = Config([{k: [] for k in KEYS}, dcfg(b_, co, p, q, 2, 4, 2), {k: [] for k in KEYS}], gc)
+        assert rel(run_plan(key, configs, [x, w, bias]), ref) <= TOL
+        gc["merge"] = [[0, 0, 1]]                  # the depthwise kernel has no bias epilogue
+        with pytest.raises(Exception):
+            schedule_with_config(key, Config(configs.op_config_lst, gc))
+        dev = [torch.from_numpy(a).cuda() for a in (x, w, bias)]
+        out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+        run_default_schedule(ops, dev + [out], stream=current_stream())
+        torch.cuda.synchronize()
+        assert rel(out.cpu().numpy(), ref) <= TOL
+    args = (2, 6, 12, 16, 12, 3, 1, 1, 1, 6)       # conv2d, groups = channels, two kernels per channel
+    register(_conv_bias, "conv2d", "bias", args, "rocm", 0)
+    key = key_of("conv2d", "bias", args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w, bias = seeded_inputs(bufs, seed=sum(args))
+    ref = oracle.bias_add_nchw_np(oracle.conv2d_nchw_c(x, w, 1, 1, 1, 6), bias)
+    s, _ = schedule_with_config(key, Config([], None))
+    assert [k.kernel for k in s.specs] == ["depthwise_f32", "bias_add_nchw_f32"]
+    assert rel(run_plan(key, Config([], None), [x, w, bias]), ref) <= TOL
+
+
 def _gemm_conv_bias(N, C, H, W, K, k, stride=1, padding=0, dilation=1, groups=1):
     from flextensor_amd.nn import gemm_conv2d_nchw
     Img = placeholder((N, C, H, W), name="Img")

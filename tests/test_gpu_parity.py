@@ -907,14 +907,17 @@ def test_depthwise_kernels_of_a_channel_fused_vs_oracle(oracle, args, th, tw, wa
     x, w = seeded_inputs(bufs, seed=sum(args))
     ref = oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8])
     b_, co, p, q = ref.shape
+    # the halo through lane shifts where the layer admits it (stride 1, rows of whole vectors)
+    shuffles = (0, 1) if (args[6] == 1 and args[8] == 1 and args[3] % 4 == 0 and tw == 4) else (0,)
     for fuse in (1, 0):
         for items in (1, 2):
-            cfgs = conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves),
-                             special=[[0], [0], [0], [items], [0], [fuse]])
-            s, _ = schedule_with_config(key, cfgs)
-            assert s.specs[-1].defines.get("MFUSE", 0) == fuse
-            out = run_plan(key, cfgs, [x, w])
-            assert rel(out, ref) <= TOL, (fuse, items)
+            for shfl in shuffles:
+                cfgs = conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves),
+                                 special=[[0], [shfl], [0], [items], [0], [fuse]])
+                s, _ = schedule_with_config(key, cfgs)
+                assert s.specs[-1].defines.get("MFUSE", 0) == fuse and s.specs[-1].defines["SHFL"] == shfl
+                out = run_plan(key, cfgs, [x, w])
+                assert rel(out, ref) <= TOL, (fuse, items, shfl)
     # borders: a constant image must give border sums with missing taps
     ones = np.ones_like(x)
     out = run_plan(key, conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves)), [ones, w])

@@ -324,8 +324,8 @@ class TileSplitSpace(SubSpace):
                         continue
                     grid = ceil_div(extent, tile)
                     padded = grid * tile
-                    if grid > 1 and (padded - extent) > max_waste * extent:
-                        continue
+                    if grid > 1 and (padded - extent) > max_waste * extent and padded - extent >= mf:
+                        continue      # (less than one MFMA block of padding is what any tiling of the axis has)
                     if grid == 1 and tile - extent >= mf:
                         continue  # a smaller tile covers the axis as well
                     ents.append([grid, w, r, mf])

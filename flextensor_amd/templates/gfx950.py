@@ -772,8 +772,9 @@ def seed_configs(op, limit=24):
     (tile aspect and MFMA edge, LDS tile extent incl. whole 3x3 windows,
     pipeline depth incl. tiles straight into LDS, K streaming when the tiles
     are fewer than the compute units, and for layers with few tiles and a
-    long K a grid-level K split sized to fill the compute units; a third of
-    the points is kept for those). The variations are entities of the op's
+    long K a grid-level K split sized to fill the compute units, or with
+    small tiles wavefront groups that share K inside the workgroup; a third
+    of the points is kept for those). The variations are entities of the op's
     space (the default config itself need not be: it may waste more of an
     edge tile than the space admits); points the templates refuse are
     dropped by the caller."""
@@ -801,7 +802,7 @@ def seed_configs(op, limit=24):
         size = t[1] * t[2] * t[3]
         if t[0] == 1:
             return size - extent < t[3]
-        return t[0] * size - extent <= 0.25 * extent
+        return t[0] * size - extent <= 0.25 * extent or t[0] * size - extent < t[3]
 
     split_seeds = []
     for (m_w, m_r, mf), (n_w, n_r, _) in shapes:
@@ -838,6 +839,26 @@ def seed_configs(op, limit=24):
                         cfg["fuse"] = [[8]]
                         cfg["reorder"] = [[1, 0, 0]]
                         split_seeds.append(cfg)
+    group_seeds = []
+    if not i8:
+        # a few small tiles and a long K (1x1 layers on a 7x7 image): one launch whose wavefront
+        # groups share K inside the workgroup and add up in LDS, with single-wavefront tiles
+        for (m_w, n_w) in ((1, 1), (2, 1), (1, 2)):
+            tm, tn = tile(view.M, m_w, 1, 16), tile(view.N, n_w, 1, 16)
+            if not (in_space(view.M, tm) and in_space(view.N, tn)) or tm[0] * tn[0] * view.groups * 2 > NUM_CUS:
+                continue
+            kps = [kp for kp in view.KP_options if kp % 16 == 0]
+            for groups in range(16 // (m_w * n_w), 1, -1):
+                if kps and (kps[0] // 16) % groups == 0:
+                    cfg = _empty_config()
+                    cfg["spatial"] = [tm, tn]
+                    cfg["reduce"] = [[groups, kps[0] // (16 * groups), 16]]
+                    cfg["unroll"] = [[3, 1]]
+                    cfg["fuse"] = [[8]]
+                    cfg["reorder"] = [[1, 1, 0]]
+                    group_seeds.append(cfg)
+                    break
+
     # spread over the variations instead of exhausting the first tile shape
     def spread(lst, n):
         if len(lst) <= n:
@@ -870,5 +891,6 @@ def seed_configs(op, limit=24):
             k += 1
         return picked
 
-    nsplit = min(len(split_seeds), limit // 3)
-    return spread_groups(out[0], out[1:], limit - nsplit) + spread(split_seeds, nsplit)
+    nsplit = min(len(split_seeds), limit // 3 - len(group_seeds))
+    return (spread_groups(out[0], out[1:], limit - nsplit - len(group_seeds)) + group_seeds +
+            spread(split_seeds, nsplit))

@@ -428,6 +428,73 @@ def test_seed_points_cover_the_decisive_knobs_and_belong_to_the_space():
     # plenty of tiles: no K split
     _, _, seeds = seeds_of(I8)
     assert all(c["reduce"][0][0] == 1 for c in seeds)
+    # 1x1 convolution on a 7x7 image, K = 832 = 52 tiles of 16: single-wavefront tiles whose 13
+    # wavefront groups share K inside the workgroup (one launch), beside the splits across workgroups
+    key = "conv2d_google38_(1, 832, 7, 7, 256, 1, 1, 0, 1, 1)_rocm(0)"
+    op, space, seeds = seeds_of(key)
+    groups = [c for c in seeds if c["reorder"] and c["reorder"][0][1] == 1]
+    assert [c["reduce"][0] for c in groups] == [[13, 4, 16], [4, 13, 16], [4, 13, 16]]
+    assert groups[0]["spatial"] == [[16, 1, 1, 16], [4, 1, 1, 16]] and len(seeds) <= 24
+    for cfg in groups:
+        assert space.subspaces["split_n_1"].index_of(cfg["spatial"][1]) >= 0
+        spec = gfx950.lower(op, cfg, None, "out", ["x", "w"])[-1]
+        assert spec.defines["WAVES_K"] == cfg["reduce"][0][0] and spec.defines["SPLITK"] == 1
+    _, _, seeds = seeds_of(CONV)
+    assert not any(c["reorder"][0][1] == 1 for c in seeds[1:])
+
+
+def test_awkward_k_may_be_zero_padded_to_wider_lds_tiles():
+    """K = 400 (16 channels x 5x5) divides into LDS tiles of 8 and 16 only; up to an eighth of zero
+    padding admits tiles of 32 .. 144. A K with a tile of 32 or more keeps its single extent."""
+    def view_of(key):
+        task = TASK_TABLE[key]
+        ops, _ = task.func(*task.args)
+        op = [o for o in flatten_graph(ops)[0] if o.kind in gfx950.GEMM_KINDS][0]
+        return op, gfx950.GemmView(op)
+    op, v = view_of("conv2d_google18_(1, 16, 14, 14, 48, 5, 1, 2, 1, 1)_rocm(0)")
+    assert (v.K, v.KP, v.KP_options) == (400, 400, [400, 416, 432, 448])
+    cfg = gfx950.default_config(op)
+    assert cfg["reduce"][0][0] * cfg["reduce"][0][1] * cfg["reduce"][0][2] == 400
+    for red, kp in (([1, 7, 64], 448), ([1, 3, 144], 432), ([13, 1, 32], 416)):
+        cfg["reduce"] = [red]
+        cfg["reorder"] = [[1, 1 if red[0] > 1 else 0, 0]]
+        spec = gfx950.lower(op, cfg, None, "out", ["x", "w"])[-1]
+        assert spec.defines["KP"] == kp and spec.defines["K"] == 400
+    cfg["reduce"], cfg["reorder"] = [[1, 4, 128]], [[1, 0, 0]]       # 512: more than an eighth of padding
+    with pytest.raises(gfx950.InvalidConfig):
+        gfx950.lower(op, cfg, None, "out", ["x", "w"])
+    assert view_of("conv2d_overfeat0_(1, 3, 192, 192, 96, 11, 4, 5, 1, 1)_rocm(0)")[1].KP_options == [368, 384]
+    assert view_of(CONV)[1].KP_options == [576] and view_of(GEMM)[1].KP_options == [1024]
+    assert view_of("conv2d_google0_(1, 3, 224, 224, 64, 7, 2, 3, 1, 1)_rocm(0)")[1].KP_options == [160]
+
+
+def test_depthwise_lowering_with_several_kernels_per_channel():
+    """kernel_fuse: lanes own patches of input planes and compute every output plane of the channel
+    (a sixth of the lanes for MobileNet's x6 stages); conv2d with one channel per group is that operator."""
+    key = "conv2d_depthwise_(8, 16, 112, 112, 6, 3, 2, 1, 1)_rocm(0)"
+    task = TASK_TABLE[key]
+    assert task.special_space["kernel_fuse"].static_entities == [[1], [0]]
+    base = gfx950.default_config(flatten_graph(task.func(*task.args)[0])[0][1])
+    def plan(fuse):
+        g = {k: [] for k in base}
+        g["inline"], g["special"] = [[1, 0]], [[0], [0], [0], [1], [0], [fuse]]
+        s, _ = schedule_with_config(key, Config([{k: [] for k in base}, base], g))
+        return s.specs[-1]
+    fused, single = plan(1), plan(0)
+    assert fused.defines["MFUSE"] == 1 and "MFUSE" not in single.defines and fused.defines["FACT"] == 6
+    assert single.grid[0] == 6 * fused.grid[0]
+    s, _ = schedule_with_config(key, Config([], None))              # the default fuses
+    assert s.specs[-1].defines.get("MFUSE") == 1
+    # one kernel per channel: the knob changes nothing
+    one = "conv2d_depthwise_(8, 512, 28, 28, 1, 3, 1, 1, 1)_rocm(0)"
+    assert "MFUSE" not in schedule_with_config(one, Config([], None))[0].specs[-1].defines
+    # conv2d with groups = input channels builds the depthwise operator and carries its knobs
+    mob = "conv2d_mobile_v21_(1, 16, 112, 112, 96, 3, 2, 1, 1, 16)_rocm(0)"
+    ops, bufs = TASK_TABLE[mob].func(*TASK_TABLE[mob].args)
+    assert ops[0].kind == "depthwise_conv2d_nchw" and ops[0].attrs["factor"] == 6 and bufs[1].shape == (96, 1, 3, 3)
+    assert "row_exchange" in TASK_TABLE[mob].special_space and "lds_pad" not in TASK_TABLE[mob].special_space
+    grp = "conv2d_grouped_(1, 1024, 14, 14, 512, 1, 1, 0, 1, 4)_rocm(0)"
+    assert TASK_TABLE[grp].func(*TASK_TABLE[grp].args)[0][0].kind == "conv2d_nchw"
 
 
 def test_schedule_ops_with_config_takes_a_flattened_op_list():

@@ -130,6 +130,12 @@ def test_tile_split_space():
                 assert new[d[0]] > cur[d[0]] and new[d[1]] < cur[d[1]]
     small = sp.TileSplitSpace(64)
     assert max(w * r * m for _, w, r, m in small.static_entities) <= 64
+    # 49 = a 7x7 image: four blocks of 16 pad 15 columns, more than a quarter of 49 but less than one
+    # block, which is what the single 64-wide tile pads as well; five blocks would pad a whole one
+    tiny = sp.TileSplitSpace(49, reps=(1, 2, 3, 4, 5, 6, 7, 8))
+    assert [4, 1, 1, 16] in tiny.static_entities and [1, 4, 1, 16] in tiny.static_entities
+    assert [2, 1, 1, 32] in tiny.static_entities and [3, 1, 1, 32] not in tiny.static_entities
+    assert all(g * w * r * m - 49 < m for g, w, r, m in tiny.static_entities)
 
 
 def test_space_container_and_generic_intra_op_space():

@@ -13,7 +13,8 @@ Operator kinds and the template each one lowers to:
                                          into the gather; or PAD=0 over a
                                          materialised padded tensor)
   gemm_int8              gemm_i8.hip
-  depthwise_conv2d_nchw  depthwise_f32.hip (direct)
+  depthwise_conv2d_nchw  depthwise_f32.hip (direct; also what conv2d_nchw builds
+                                         for one input channel per group)
   zero_pad2d             elementwise.hip   (only when not inlined)
 
 Meaning of the config keys: see flextensor_amd/space.py.

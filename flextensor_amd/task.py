@@ -125,6 +125,9 @@ def _attach_default_knobs(task):
         return
     if kind == "conv2d_nchw" and len(task.args) > 9 and task.args[9] > 1 and task.args[1] == task.args[9]:
         kind = "depthwise_conv2d_nchw"        # one input channel per group: nn.conv2d_nchw builds that operator
+    elif kind == "conv2d_nchw" and len(task.args) > 9 and \
+            (task.args[0], task.args[5], task.args[6], task.args[7], task.args[9]) == (1, 1, 1, 0, 1):
+        kind = "pointwise_conv2d_nchw"        # one image, 1x1, stride 1, no padding, one group
     for key, knobs in special_knobs(kind).items():
         if key not in task.special_space:
             task.set_specific_space(key, "enum", knobs)

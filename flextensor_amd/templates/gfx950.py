@@ -138,6 +138,10 @@ class GemmView(object):
             self.groups = groups
             self.conv = dict(CB=b, CG=groups, CC=c * groups, CH=h, CW=w, CR=r, CS=s, CP=p, CQ=q,
                              **_conv_steps(a))
+            # one image, 1x1 kernel, stride 1, no padding: O [K][H*W] = W [K][C] x X [C][H*W] in the
+            # tensors' own layouts, a plain GEMM whose B rows load as 16-byte vectors
+            self.pointwise = (b == 1 and groups == 1 and r == 1 and s == 1 and tuple(a["stride"]) == (1, 1)
+                              and tuple(a["padding"]) == (0, 0))
         elif kind == "col_gemm":
             # the GEMM stage of an im2col convolution: one [Mg,K] x [K,N] product per group.
             # With the column matrix read through (inlined) it is the implicit GEMM over the
@@ -257,6 +261,9 @@ SPECIAL_DEFAULTS = {
     "row_exchange": [0],
     # depthwise with several kernels per input channel: 1 = a lane computes its patch for all of them
     "kernel_fuse": [1],
+    # 1x1 convolution, stride 1, no padding, one image: 1 = the GEMM addressing mode (the image is
+    # the B matrix as it lies in memory, rows load as 16-byte vectors), 0 = the gather of the general case
+    "image_as_matrix": [1],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -273,6 +280,11 @@ PIPELINE = {1: (1, 1), 2: (2, 1), 3: (2, 2), 4: (2, 3), 5: (2, 1), 6: (2, 1), 7:
 def special_knobs(kind):
     """Enumerated knobs a task of this operator kind carries by default; they
     are attached with Task.set_specific_space and searched at graph level."""
+    if kind == "pointwise_conv2d_nchw":
+        # a 1x1 / stride 1 / unpadded convolution over one image (the task tells: the operator kind
+        # is conv2d_nchw like any other convolution's)
+        return {"lds_pad": [[-1, -1], [4, -1], [4, 8], [4, 4], [0, 0], [8, -1], [-1, 0]],
+                "image_as_matrix": [[1], [0]]}
     if kind in ("gemm", "conv2d_nchw", "batch_gemm", "col_gemm"):
         return {"lds_pad": [[-1, -1], [4, -1], [4, 8], [4, 4], [0, 0], [8, -1], [-1, 0]]}
     if kind == "gemm_int8":
@@ -304,6 +316,9 @@ def _one(config, key, n, what):
 def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None,
                 through=(), merged_out=None):
     view = GemmView(op, col_inlined="im2col_nchw" in through)
+    if getattr(view, "pointwise", False) and int(_special(special, "image_as_matrix")[0]) \
+            and bias_name is None and merged_out is None:
+        view.mode = 0        # A = weight [K][C], B = image [C][H*W], C = output [K][H*W]
     if bias_name is not None and view.mode != 1 and op.kind != "col_gemm":
         raise InvalidConfig("only the convolution has a bias epilogue")
     if merged_out is not None and not (op.kind == "col_gemm" and merged_out == "col2img_nchw"):
@@ -491,8 +506,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         a_name, b_name = in_names[1], in_names[0]
     else:
         a_name, b_name = in_names[0], in_names[1]
-        if op.kind == "col_gemm":
-            a_name, b_name = in_names[1], in_names[0]      # A = weight, B = stored columns
+        if op.kind in ("col_gemm", "conv2d_nchw"):
+            a_name, b_name = in_names[1], in_names[0]      # A = weight, B = stored columns / the image
         if view.groups > 1:
             D.update(CG=view.groups)      # batched GEMM
     if splitk > 1:

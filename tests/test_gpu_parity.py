@@ -780,6 +780,35 @@ def test_conv2d_vs_oracle(oracle, args, kn):
         assert rel(out, oracle.conv2d_nchw_np(x, w, st, pd, dl, g)) <= TOL
 
 
+@pytest.mark.parametrize("args,kn", [
+    ((1, 64, 14, 14, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, st=3)),         # 196 pixels: 16-byte image rows
+    ((1, 64, 14, 14, 96, 1, 1, 0, 1, 1), dict(wm=1, rm=1, wn=4, rn=1, mf=16, bk=64, st=8, ls=2)),   # tiles straight into LDS
+    ((1, 48, 7, 7, 40, 1, 1, 0, 1, 1), dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=16, st=2, sk=3, wk=1)),  # 49 pixels: single floats
+    ((1, 48, 13, 13, 24, 1, 1, 0, 2, 1), dict(wm=1, rm=1, wn=2, rn=1, mf=16, bk=16, st=5)),         # dilation has no meaning at 1x1
+    ((1, 72, 28, 28, 64, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=72, st=3, ks=1)),   # K streaming
+])
+def test_pointwise_conv2d_over_one_image_as_a_gemm(oracle, args, kn):
+    """1x1 / stride 1 / unpadded convolution of one image: O [K][H*W] = W [K][C] x X [C][H*W] in the
+    tensors' own layouts. image_as_matrix 1 lowers it in the GEMM addressing mode, 0 as the gather."""
+    register(conv2d, "conv2d", "t", args, "rocm", 0)
+    key = key_of("conv2d", "t", args)
+    assert list(TASK_TABLE[key].special_space) == ["lds_pad", "image_as_matrix"]
+    ops, bufs = TASK_TABLE[key].func(*args)
+    x, w = seeded_inputs(bufs, seed=sum(args))
+    nb, c, h, wd, ko, ks, st, pd, dl, g = args
+    ref = oracle.conv2d_nchw_c(x, w, st, pd, dl, g)
+    cfg = gcfg(ko, h * wd, c, **kn)
+    for flag in (1, 0):
+        for inline in ([1, 0], [0, 0]):
+            cfgs = conv_cfgs(cfg, inline, special=[[-1, -1], [flag]])
+            s, _ = schedule_with_config(key, cfgs)
+            assert s.specs[-1].defines["MODE"] == (0 if flag else 1)
+            assert rel(run_plan(key, cfgs, [x, w]), ref) <= TOL, (flag, inline)
+    s, _ = schedule_with_config(key, Config([], None))               # the default is the GEMM mode
+    assert s.specs[-1].defines["MODE"] == 0
+    assert rel(run_plan(key, Config([], None), [x, w]), ref) <= TOL
+
+
 @pytest.mark.parametrize("args", [
     (2, 24, 10, 10, 24, 3, 1, 1, 1, 24),          # groups = channels, one kernel per channel
     (1, 8, 12, 16, 48, 3, 2, 1, 1, 8),            # six kernels per channel, stride 2 (a MobileNet stage)

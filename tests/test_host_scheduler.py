@@ -12,6 +12,7 @@ from flextensor_amd.scheduler import flatten_graph, schedule, schedule_with_conf
 from flextensor_amd.space import generate_space_intra_op
 from flextensor_amd.task import TASK_TABLE, Task, register_task, gemm, conv2d
 from flextensor_amd.templates import gfx950
+from flextensor_amd.tuned import lookup
 from flextensor_amd.utils import Config
 
 GEMM = "gemm_gemm_(1024, 1024, 1024)_rocm(0)"
@@ -466,6 +467,37 @@ def test_awkward_k_may_be_zero_padded_to_wider_lds_tiles():
     assert view_of("conv2d_overfeat0_(1, 3, 192, 192, 96, 11, 4, 5, 1, 1)_rocm(0)")[1].KP_options == [368, 384]
     assert view_of(CONV)[1].KP_options == [576] and view_of(GEMM)[1].KP_options == [1024]
     assert view_of("conv2d_google0_(1, 3, 224, 224, 64, 7, 2, 3, 1, 1)_rocm(0)")[1].KP_options == [160]
+
+
+def test_pointwise_convolution_of_one_image_lowers_in_the_gemm_mode():
+    """1x1 / stride 1 / unpadded / one image: the image is the B matrix as it lies in memory; the task
+    carries the knob that chooses between that and the general gather, other convolutions do not."""
+    key = "conv2d_yolo10_(1, 1024, 14, 14, 512, 1, 1, 0, 1, 1)_rocm(0)"
+    assert list(TASK_TABLE[key].special_space) == ["lds_pad", "image_as_matrix"]
+    s, _ = schedule_with_config(key, Config([], None))
+    d = s.specs[-1].defines
+    assert (d["MODE"], d["BV"], d["M"], d["N"], d["K"]) == (0, 4, 512, 196, 1024) and "CH" not in d
+    assert [a[1] for a in s.specs[-1].args[:3]] == ["in1", "in0", "out"]  # A = weight, B = image
+    cfg = lookup(key)
+    g = dict(cfg.graph_config)
+    g["special"] = [list((g.get("special") or [[-1, -1]])[0]), [0]]
+    d = schedule_with_config(key, Config(cfg.op_config_lst, g))[0].specs[-1].defines
+    assert d["MODE"] == 1 and d["BV"] == 1 and d["CH"] == 14
+    for other in (CONV, CONV1x1, "conv2d_res5_(64, 256, 56, 56, 512, 1, 2, 0, 1, 1)_rocm(0)"):
+        assert list(TASK_TABLE[other].special_space) == ["lds_pad"]       # 3x3; batch 8; stride 2
+        assert schedule_with_config(other, Config([], None))[0].specs[-1].defines["MODE"] == 1
+    # a bias runs in the convolution's epilogue, which the GEMM mode does not have
+    from flextensor_amd.nn import conv2d_nchw
+    from flextensor_amd.te import placeholder
+
+    def with_bias():
+        x, w, b = placeholder((1, 32, 14, 14), name="Img"), placeholder((48, 32, 1, 1), name="W"), placeholder((48,), name="b")
+        out = conv2d_nchw(x, w, b)
+        return [out.op], [x, w, b, out]
+    t = Task("conv2d", "pw_bias", with_bias, (), "rocm", 0)
+    register_task(t, override=True)
+    kernels = schedule_with_config(t.key, Config([], None))[0].specs
+    assert kernels[-1].defines["MODE"] == 1 and kernels[-1].defines.get("HAS_BIAS") == 1
 
 
 def test_depthwise_lowering_with_several_kernels_per_channel():

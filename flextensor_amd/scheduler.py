@@ -725,9 +725,14 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
         if kwargs.get("warm_start", True):
             from .tuned import lookup
             shipped = lookup(task_key, similar=True)
-            if shipped is not None and shipped.graph_config and \
-                    len(shipped.graph_config.get("special") or []) == len(task.special_space):
-                configs = Config([], dict(shipped.graph_config))
+            if shipped is not None and shipped.graph_config:
+                # an entry written before a knob existed leaves it out: it takes the knob's default
+                graph = dict(shipped.graph_config)
+                have = list(graph.get("special") or [])
+                names = list(task.special_space)
+                if len(have) <= len(names) and all(n in gfx950.SPECIAL_DEFAULTS for n in names[len(have):]):
+                    graph["special"] = have + [list(gfx950.SPECIAL_DEFAULTS[n]) for n in names[len(have):]]
+                    configs = Config([], graph)
 
     schedulers = []
     try:

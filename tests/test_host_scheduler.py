@@ -326,6 +326,26 @@ def test_schedule_searching_finds_known_optimum_and_roundtrips():
     assert s2.describe() == s.describe()
 
 
+def test_warm_start_takes_an_entry_written_before_a_knob_existed():
+    """The shipped entry of a 1x1 layer pinned to the gather has both knobs, most have lds_pad only:
+    either way the operator search runs under the entry's graph config, missing knobs at their defaults."""
+    seen = {}
+
+    def cost(task_key, cfg, op_pos, number):
+        s, _ = schedule_with_config(task_key, cfg, op_pos=op_pos)
+        if op_pos is not None:
+            seen.setdefault(task_key, set()).add(s.specs[-1].defines["MODE"])
+        return 1.0 + 1e-4 * s.specs[-1].grid[0]
+
+    gather = "conv2d_yolo8_(1, 512, 28, 28, 512, 1, 1, 0, 1, 1)_rocm(0)"      # special [[..], [0]]
+    older = "conv2d_yolo10_(1, 1024, 14, 14, 512, 1, 1, 0, 1, 1)_rocm(0)"     # special [[..]]
+    assert len(lookup(gather).graph_config["special"]) == 2 and len(lookup(older).graph_config["special"]) == 1
+    for key in (gather, older):
+        np.random.seed(2)
+        schedule(key, op_trial=2, graph_trial=1, parallel=2, method="random", evaluator=cost, verbose=False)
+    assert seen[gather] == {1} and seen[older] == {0}
+
+
 def test_schedule_random_method_and_conv_graph():
     np.random.seed(1)
     calls = []

@@ -208,6 +208,26 @@ def test_depthwise_vs_torch(oracle):
         assert rel(oracle.depthwise_nchw_np(x, wt, st, p, d), ref) < 1e-12
 
 
+def test_identities_the_special_lowerings_rest_on(oracle):
+    """A convolution with one input channel per group is the depthwise operator on the same weight
+    bytes, term for term (so bit for bit); a 1x1 stride-1 unpadded convolution of one image is the
+    product W [K][C] x X [C][H*W], summed over c in the same order."""
+    rng = np.random.default_rng(11)
+    for (n, c, h, w, f, k, st, p, d) in [(2, 6, 9, 11, 1, 3, 1, 1, 1), (1, 4, 12, 16, 6, 3, 2, 1, 1),
+                                         (2, 5, 9, 11, 2, 3, 1, 1, 2)]:
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (c, f, k, k)).astype(np.float32)
+        grouped = oracle.conv2d_nchw_c(x, wt.reshape(c * f, 1, k, k), st, p, d, c)
+        assert np.array_equal(grouped, oracle.depthwise_nchw_c(x, wt, st, p, d))
+    for (c, h, w, ko) in [(64, 14, 14, 96), (48, 7, 7, 40)]:
+        x = rng.uniform(-1, 1, (1, c, h, w)).astype(np.float32)
+        wt = rng.uniform(-1, 1, (ko, c, 1, 1)).astype(np.float32)
+        conv = oracle.conv2d_nchw_c(x, wt, 1, 0, 1, 1)
+        prod = oracle.gemm_f32_c(wt.reshape(ko, c), x.reshape(c, h * w))
+        assert np.array_equal(conv.reshape(ko, h * w), prod)
+        assert rel(conv.reshape(ko, h * w), wt.reshape(ko, c).astype(np.float64) @ x.reshape(c, h * w).astype(np.float64)) < 1e-6
+
+
 def test_gemm_f32(oracle, gold):
     a, b = gold["gemm_a"], gold["gemm_b"]
     assert rel(oracle.gemm_f32_c(a, b), gold["gemm_c"]) < 1e-6

@@ -43,13 +43,7 @@ thread_local std::string g_err;
     } while (0)
 
 int launch_one(const ftr_launch_desc_t &d, hipStream_t s) {
-    if (!d.mod) return fail("ftr_launch: null module");
-    if (!d.args) return fail("ftr_launch: null argument array");
-    for (int i = 0; i < 3; ++i)
-        if (d.grid[i] == 0 || d.block[i] == 0)
-            return fail("ftr_launch: zero grid/block extent in dim %d", i);
-    if ((unsigned long long)d.block[0] * d.block[1] * d.block[2] > 1024ull)
-        return fail("ftr_launch: more than 1024 threads per workgroup");
+    if (ftr_internal_check_desc(&d)) return 1;
     FTR_HIP(hipModuleLaunchKernel(d.mod->func, d.grid[0], d.grid[1], d.grid[2],
                                   d.block[0], d.block[1], d.block[2],
                                   d.lds_bytes, s, d.args, nullptr));
@@ -57,6 +51,17 @@ int launch_one(const ftr_launch_desc_t &d, hipStream_t s) {
 }
 
 }  // namespace
+
+int ftr_internal_check_desc(const ftr_launch_desc_t *d) {
+    if (!d->mod) return fail("ftr_launch: null module");
+    if (!d->args) return fail("ftr_launch: null argument array");
+    for (int i = 0; i < 3; ++i)
+        if (d->grid[i] == 0 || d->block[i] == 0)
+            return fail("ftr_launch: zero grid/block extent in dim %d", i);
+    if ((unsigned long long)d->block[0] * d->block[1] * d->block[2] > 1024ull)
+        return fail("ftr_launch: more than 1024 threads per workgroup");
+    return 0;
+}
 
 int ftr_internal_fail(const char *fmt, ...) {
     char buf[4096];
@@ -150,11 +155,10 @@ int ftr_module_load(const void *code, size_t size, const char *kernel_name,
                     hipGetErrorString(e));
     }
     // set-up time is also when the static workspace of this device is looked
-    // up, so that ftr_launch_seq_static_ws has nothing left to resolve later
-    if (ftr_internal_static_ws(nullptr)) {
-        (void)hipModuleUnload(m);
-        return 1;
-    }
+    // up, so that ftr_launch_seq_static_ws normally has nothing left to resolve.
+    // Only that entry point needs the array: a device on which the look-up fails
+    // still loads modules, and ftr_launch_seq_static_ws reports the failure.
+    (void)ftr_internal_static_ws(nullptr);
     ftr_module *mod = new ftr_module{m, f};
     *out = mod;
     return 0;

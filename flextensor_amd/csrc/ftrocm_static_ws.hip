@@ -64,7 +64,9 @@ extern "C" int ftr_launch_seq_static_ws(const ftr_launch_desc_t *seq, int n, con
                                         int nbinds, void *stream) {
     if (!seq || n < 1 || nbinds < 0 || (nbinds > 0 && !binds))
         return ftr_internal_fail("ftr_launch_seq_static_ws: bad argument");
-    // validate everything before anything is enqueued or written
+    // validate everything, launch descriptors included, before anything is enqueued or written
+    for (int i = 0; i < n; ++i)
+        if (ftr_internal_check_desc(&seq[i])) return 1;
     for (int b = 0; b < nbinds; ++b) {
         const ftr_ws_bind_t &w = binds[b];
         if (w.launch < 0 || w.launch >= n || w.arg < 0)

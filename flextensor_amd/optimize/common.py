@@ -7,6 +7,7 @@ plain default-schedule kernels of the same task on the device, which is what
 the reference's ``check_result`` does with the default llvm build, and runs
 the static check of the kernels' assembly (isa_check).
 """
+import os
 import sys
 
 from ..measure import get_measurer
@@ -41,7 +42,6 @@ def test(task_key, configs, dev_id=None, rpc_info=None, check_result=False):
         print("Test correctness...", "passed!" if ok else "failed!", "metric", metric)
         # and the assembly: no read of an MFMA's result before the matrix core has written it
         from .. import isa_check
-        import os
         if os.path.exists(isa_check.HIPCC):
             early = isa_check.check_plan(s)
             print("Test instruction stream...", "passed!" if not early else "failed! %s" % (early[:2],))

@@ -42,7 +42,7 @@ def able_inline(op, down_graph):
 
 # stage kind -> producer kinds whose kernel can take the stage over
 MERGE_RULES = {
-    "bias_add_nchw": ("conv2d_nchw",),            # bias in the convolution's epilogue
+    "bias_add_nchw": ("conv2d_nchw", "depthwise_conv2d_nchw"),   # bias in the convolution's epilogue
     "bias_add_ghw": ("col_gemm",),                # the same for the GEMM of an im2col convolution
     "col2img_nchw": ("col_gemm", "bias_add_ghw"),  # the GEMM stores NCHW itself
 }

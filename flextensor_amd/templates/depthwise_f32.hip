@@ -31,6 +31,8 @@
 // above and below between lanes through a wavefront-private LDS window: no
 // barrier, no halo re-reads from memory except the one row either side of
 // the span; the padding rows arrive as the zeros of out-of-range loads.
+// HAS_BIAS = 1 adds a per-output-channel bias (ops.py:673-677) to every
+// result in the store, from a fourth argument; all three variants take it.
 // Shape constants: CB batch, CC channels, CH x CW input, CR x CS kernel,
 // STRH/STRW, PADH/PADW, DILH/DILW (rows / columns), FACT, CP x CQ output.
 
@@ -66,6 +68,16 @@
 #else
 #define MFUSE 0
 #endif
+#ifdef FT_HAS_BIAS
+#define HAS_BIAS FT_HAS_BIAS
+#else
+#define HAS_BIAS 0
+#endif
+#if HAS_BIAS
+#define BIAS_PARAM , const float* __restrict__ Bs
+#else
+#define BIAS_PARAM
+#endif
 #define CB FT_CB
 #define CC FT_CC
 #define CH FT_CH
@@ -96,13 +108,18 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 /* 128-bit path: a convolution with stride 1 or 2 along W whose output rows
  * are 1/STRW of the input rows and whose rows keep 16-byte alignment; the
  * 4 * STRW input columns from the patch's first output column on come in as
- * STRW vectors (of a ragged last patch they may run into the next row: those
- * elements only feed outputs that are not stored). */
+ * STRW vectors. Of a ragged last patch (CQ % 4 != 0) they run into the next
+ * row. The last stored output column, CQ - 1, reads up to input column
+ * CW - STRW + (CS - 1) * DILW - PADW: when that stays below CW the elements
+ * from the next row only feed outputs that are not stored; otherwise columns
+ * CW and beyond are padding that a stored output does read, and every vector
+ * element whose column is not below CW is replaced by zero (VEC_CLIP). */
 #if (TW == 4) && (STRW <= 2) && (CW % 4 == 0) && (CQ * STRW == CW) && (PADW + 4 * STRW <= IW_T)
 #define VEC_IN 1
 #else
 #define VEC_IN 0
 #endif
+#define VEC_CLIP (VEC_IN && (CQ % 4 != 0) && ((CS - 1) * DILW - PADW >= STRW))
 #define NVEC STRW
 #if (TW == 4) && (CQ % 4 == 0)
 #define VEC_OUT 1
@@ -130,7 +147,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O)
+                   float* __restrict__ O BIAS_PARAM)
 {
     __shared__ __attribute__((aligned(16))) float sx[LDSP * PS];
     __shared__ __attribute__((aligned(16))) float sw[LDSP * 12];     /* 3 taps + 1 pad per kernel row */
@@ -190,6 +207,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                 for (int t = 0; t < 3; ++t)
                     acc[j] += in[j + t] * w[t];
         }
+#if HAS_BIAS
+        acc += Bs[plane % (CC * FACT)];
+#endif
 #if NT_STORE
         __builtin_nontemporal_store(acc, &O4[(size_t)plane * PLANE4 + rem]);
 #else
@@ -219,10 +239,14 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O)
+                   float* __restrict__ O BIAS_PARAM)
 {
-    /* window chunk ro * Q4 + col of a wavefront holds (row r0 - 1 + ro, chunk col) of its plane */
-    __shared__ __attribute__((aligned(16))) float sx[(NT / 64) * WIN * 4];
+    /* window chunk ro * Q4 + col of a wavefront holds (row r0 - 1 + ro, chunk col) of its plane.
+     * Idle lanes (LPW .. 63) read the chunk their own lane number points at, like the busy ones:
+     * 64 consecutive chunks per read, which the LDS serves without a bank conflict (an idle lane
+     * parked on one fixed chunk shares its banks with a busy lane of the same pass). What they
+     * read, from the next wavefront's window or the slack behind the last one, is never used. */
+    __shared__ __attribute__((aligned(16))) float sx[((NT / 64) * WIN + 64) * 4];
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, X_BYTES, 0x00020000);
     const int lane = threadIdx.x & 63;
@@ -257,6 +281,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #pragma unroll
     for (int t = 0; t < 9; ++t)
         w[t] = Wt[ch * 9 + t];
+#if HAS_BIAS
+    const float bias = Bs[ch];
+#endif
 
     /* ---- rows change lanes through the window -------------------------------- */
     if (lane < LPW) {
@@ -275,7 +302,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
     const bool left = col == 0, right = col == Q4 - 1;
 #pragma unroll
     for (int i = 0; i < WX; ++i) {
-        const float* mid = &win[((1 + i * RPI) * Q4 + (lane < LPW ? lane : 0)) * 4];   /* idle lanes stay inside the window */
+        const float* mid = &win[((1 + i * RPI) * Q4 + lane) * 4];
         f32x4 acc = (f32x4)(0.0f);
 #pragma unroll
         for (int r = 0; r < 3; ++r) {
@@ -296,6 +323,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
                 for (int t = 0; t < 3; ++t)
                     acc[c] += in[c + t] * w[r * 3 + t];
         }
+#if HAS_BIAS
+        acc += bias;                     /* FACT == 1: the plane's channel is its output channel */
+#endif
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), ro, (int)vo[i], 0, ST_AUX);
     }
 }
@@ -314,11 +344,15 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O)
+                   float* __restrict__ O BIAS_PARAM)
 {
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(Wt), 0, W_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, O_BYTES, 0x00020000);
+#if HAS_BIAS
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(Bs), 0, CC * FACT * 4, 0x00020000);
+    float bias[IPL][FM];
+#endif
 
     /* A lane works on IPL patches, NT lanes (LPW per wavefront) apart, so that a
      * workgroup covers one contiguous run of IPL * (lanes that carry work)
@@ -371,6 +405,10 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         for (int m = 0; m < FM; ++m) {
             /* the kernel's CR*CS taps: 128-bit loads (dword-aligned is enough for buffer loads) and a tail */
             const unsigned wo = live[k] ? (unsigned)((co + m) * (CR * CS)) * 4u : OOB;
+#if HAS_BIAS
+            bias[k][m] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                rb, (int)(live[k] ? (unsigned)(co + m) * 4u : OOB), 0, 0));
+#endif
             float wflat[(CR * CS + 3) / 4 * 4];
 #pragma unroll
             for (int t = 0; t + 4 <= CR * CS; t += 4) {
@@ -447,9 +485,14 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #elif VEC_IN
             {
 #pragma unroll
-                for (int j = 0; j < IW_T; ++j)
+                for (int j = 0; j < IW_T; ++j) {
                     in[j] = (j >= PADW && j < PADW + 4 * NVEC) ? rows[k][y][((j - PADW) >> 2) % NVEC][(j - PADW) & 3]
                                                                : halo[k][y][j];
+#if VEC_CLIP
+                    /* a ragged last patch: vector elements beyond the row's end are the right padding */
+                    if (j >= PADW && j < PADW + 4 * NVEC && tw[k] * (TW * STRW) + (j - PADW) >= CW) in[j] = 0.0f;
+#endif
+                }
             }
 #else
 #pragma unroll
@@ -475,6 +518,10 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #pragma unroll
         for (int i = 0; i < TH; ++i) {
             const bool row_ok = live[k] && (CP % TH == 0 || oh0[k] + i < CP);
+#if HAS_BIAS
+#pragma unroll
+            for (int j = 0; j < TW; ++j) acc[i][j] += bias[k][m];
+#endif
 #if VEC_OUT
             f32x4 v;
             v[0] = acc[i][0]; v[1] = acc[i][1]; v[2] = acc[i][2]; v[3] = acc[i][3];

@@ -264,6 +264,12 @@ SPECIAL_DEFAULTS = {
     # 1x1 convolution, stride 1, no padding, one image: 1 = the GEMM addressing mode (the image is
     # the B matrix as it lies in memory, rows load as 16-byte vectors), 0 = the gather of the general case
     "image_as_matrix": [1],
+    # K streaming: 1 = the arrival count and the look at the counter are a device-scope
+    # release / acquire (what the memory model asks for; costs an L2 write-back and invalidate per
+    # hand-off, +4.5 % on the 8x256x14x14 benchmark layer), 0 = relaxed device-scope atomics behind
+    # an explicit wait for the slot stores (the measured trade-off the shipped entries use). Not in
+    # the searched knobs: a task opts in with set_specific_space("sk_fenced", "enum", [[1]])
+    "sk_fenced": [0],
 }
 
 # unroll entity [[depth, 1]] -> (LDS stages, prefetch distance in tiles);
@@ -530,6 +536,8 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         if xcd:
             ngrid = ceil_div(ngrid, NUM_XCD) * NUM_XCD   # renumbering by XCD needs whole rounds
         D.update(SK_PER=per)
+        if int(_special(special, "sk_fenced")[0]):
+            D.update(SK_FENCED=1)
         grid = (ngrid, 1, 1)
         workspace = {out_name + "_parts": ((ngrid * 2 * nt * nacc,), "float32"),
                      out_name + "_count": ((gm * gn * view.groups,), "int32")}
@@ -543,7 +551,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     return specs
 
 
-def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=False):
+def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=False, bias_name=None):
     sp = _one(config, "spatial", 4, op.kind)
     th, tw = int(sp[2][3]), int(sp[3][3])
     if int(sp[0][3]) != 1 or int(sp[1][3]) != 1:
@@ -582,6 +590,11 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
     ldsp = int(_special(special, "lds_planes")[0])
     nt_mode = int(_special(special, "nt_store")[0])     # bit 0: non-temporal stores, bit 1: non-temporal loads
     steps = dict(STRH=st_h, STRW=st_w, PADH=pad_h, PADW=pad_w, DILH=dl_h, DILW=dl_w)
+    args = [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)]
+    if bias_name is not None:
+        # the bias stage merged into the kernel: added to every result in the store (ops.py:673-677)
+        steps["HAS_BIAS"] = 1
+        args.append(("buf", bias_name))
     if ldsp:
         # plane-staged variant: whole planes through LDS in copy order; the lane patch knobs do not apply
         if not (st_h == st_w == 1 and dl_h == dl_w == 1 and r_ext == 3 and s_ext == 3 and pad_h == pad_w == 1
@@ -592,8 +605,7 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=0, LDSP=ldsp,
                  CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=1, CP=p, CQ=q, **steps)
         return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (ceil_div(b * cout, ldsp), 1, 1),
-                           (nt, 1, 1),
-                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
+                           (nt, 1, 1), args)]
     wx = int(_special(special, "row_exchange")[0])
     if wx:
         # row-exchange variant: a wavefront owns rpi * wx rows of one plane (rpi whole rows per load
@@ -611,13 +623,12 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         if rpi * 4 < rpi_max * 3:
             rpi = rpi_max         # too few lanes would carry work: ragged last span instead
         rows = rpi * wx
-        if waves * (rows + 2) * q4 * 16 > LDS_BYTES:
+        if (waves * (rows + 2) * q4 + 64) * 16 > LDS_BYTES:      # 64 chunks of slack for the idle lanes' reads
             raise InvalidConfig("row-exchange windows do not fit the LDS")
         D = dict(NT=nt, TH=th, TW=tw, NT_STORE=nt_mode & 1, NT_LOAD=nt_mode >> 1, SHFL=0, WX=wx, WXR=rpi,
                  CB=b, CC=c, CH=h, CW=w, CR=r_ext, CS=s_ext, FACT=1, CP=p, CQ=q, **steps)
         return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D,
-                           (ceil_div(b * cout * ceil_div(h, rows), waves), 1, 1), (nt, 1, 1),
-                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
+                           (ceil_div(b * cout * ceil_div(h, rows), waves), 1, 1), (nt, 1, 1), args)]
     shfl = int(_special(special, "halo_shfl")[0])
     tiles_w = ceil_div(q, tw)
     if shfl:
@@ -633,9 +644,7 @@ def _lower_depthwise(op, config, special, out_name, in_names, materialized_pad=F
         D.update(IPL=ipl)
     if fm > 1:
         D.update(MFUSE=1)
-    return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1),
-                       (nt, 1, 1),
-                       [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])]
+    return [KernelSpec("depthwise_f32.hip", "depthwise_f32", D, (grid_x, 1, 1), (nt, 1, 1), args)]
 
 
 def _lower_pad(op, out_name, in_names):
@@ -702,18 +711,18 @@ def lower(op, config, special, out_name, in_names, materialized_pad=False, bias_
     if op.kind in GEMM_KINDS:
         return _lower_gemm(op, config, special, out_name, in_names, materialized_pad, bias_name,
                            through, merged_out)
-    if bias_name is not None:
-        raise InvalidConfig("operator kind %s has no bias epilogue" % op.kind)
     if merged_out is not None:
         raise InvalidConfig("operator kind %s takes no merged stage" % op.kind)
+    if op.kind == "depthwise_conv2d_nchw":
+        return _lower_depthwise(op, config, special, out_name, in_names, materialized_pad, bias_name)
+    if bias_name is not None:
+        raise InvalidConfig("operator kind %s has no bias epilogue" % op.kind)
     if op.kind == "im2col_nchw":
         return _lower_im2col(op, out_name, in_names, materialized_pad)
     if op.kind == "col2img_nchw":
         return _lower_col2img(op, out_name, in_names)
     if op.kind in ("bias_add_nchw", "bias_add_ghw"):
         return _lower_bias(op, out_name, in_names)
-    if op.kind == "depthwise_conv2d_nchw":
-        return _lower_depthwise(op, config, special, out_name, in_names, materialized_pad)
     if op.kind == "zero_pad2d":
         return _lower_pad(op, out_name, in_names)
     raise InvalidConfig("no gfx950 template for operator kind %s" % op.kind)
@@ -907,6 +916,7 @@ def seed_configs(op, limit=24):
             k += 1
         return picked
 
-    nsplit = min(len(split_seeds), limit // 3 - len(group_seeds))
-    return (spread_groups(out[0], out[1:], limit - nsplit - len(group_seeds)) + group_seeds +
-            spread(split_seeds, nsplit))
+    group_seeds = group_seeds[:max(limit // 3, 0)]
+    nsplit = max(0, min(len(split_seeds), limit // 3 - len(group_seeds)))
+    return (spread_groups(out[0], out[1:], max(limit - nsplit - len(group_seeds), 1)) + group_seeds +
+            spread(split_seeds, nsplit))[:max(limit, 1)]

@@ -168,7 +168,9 @@ typedef struct ftr_ws_bind {
  * fit. The array is one per GPU and keeps the previous call's contents: ask
  * for zero where a kernel relies on zeros. Calls that overlap in time on one
  * GPU (two streams, two threads) race on it. The array's address is resolved
- * per device at ftr_module_load time. */
+ * once per device: at the first ftr_module_load on that device, or, for a
+ * device on which no module was loaded through this library yet, at the
+ * first call of this entry point. */
 int ftr_launch_seq_static_ws(const ftr_launch_desc_t *seq, int n,
                              const ftr_ws_bind_t *binds, int nbinds,
                              void *stream);

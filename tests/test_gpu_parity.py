@@ -25,6 +25,7 @@ from flextensor_amd.task import (TASK_TABLE, Task, register, gemm, gemm_int8, co
                                  depthwise_conv2d)
 from flextensor_amd.nn import gemm as op_gemm  # noqa: E402
 from flextensor_amd.te import placeholder  # noqa: E402
+from flextensor_amd.templates.gfx950 import special_knobs  # noqa: E402
 from flextensor_amd.utils import Config, ceil_div  # noqa: E402
 
 TOL = 1e-5
@@ -268,6 +269,20 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
     assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[0], outs[3])
     assert int(func.scratch["out_count"].abs().sum().item()) == 0
     func.close()
+    # the hand-off as a device-scope release / acquire on the counter (a task opts in): the same
+    # sums in the same order, so the same bits
+    TASK_TABLE[key].set_specific_space("sk_fenced", "enum", [[1]])
+    try:
+        g = {k: [] for k in KEYS}
+        g["special"] = [[-1, -1], [1]]
+        assert list(TASK_TABLE[key].special_space)[-1] == "sk_fenced"
+        fenced = Config(cfg.op_config_lst, g)
+        s2, _ = schedule_with_config(key, fenced)
+        assert s2.specs[-1].defines["SK_FENCED"] == 1 and "SK_FENCED" not in s.specs[-1].defines
+        a, b = seeded_inputs(bufs, seed=1)
+        assert np.array_equal(run_plan(key, fenced, [a, b]), outs[0])
+    finally:
+        TASK_TABLE[key].special_space.pop("sk_fenced", None)
 
 
 @pytest.mark.parametrize("M,K,N,kn,pad", [
@@ -456,25 +471,37 @@ def _depthwise_bias(N, C, H, W, factor, k, stride=1, padding=0, dilation=1):
 
 
 def test_depthwise_and_one_channel_groups_with_bias(oracle):
-    """[Padding, depthwise, bias] (flextensor/nn/ops.py:673-677): the bias runs as its own kernel
-    behind the depthwise kernel; conv2d_nchw with groups = channels and a bias builds the same graph."""
+    """[Padding, depthwise, bias] (flextensor/nn/ops.py:673-677): the bias is added in the stores of
+    the depthwise kernel (merge 1, the default) or runs as its own kernel behind it (merge 0), in
+    every variant of the kernel; conv2d_nchw with groups = channels and a bias builds the same graph."""
     for args in ((2, 6, 12, 16, 1, 3, 1, 1, 1), (1, 4, 14, 16, 6, 3, 2, 1, 1)):
         register(_depthwise_bias, "conv2d", "dw_bias", args, "rocm", 0)
         key = key_of("conv2d", "dw_bias", args)
+        for name, knobs in special_knobs("depthwise_conv2d_nchw").items():
+            TASK_TABLE[key].set_specific_space(name, "enum", knobs)
         ops, bufs = TASK_TABLE[key].func(*args)
         x, w, bias = seeded_inputs(bufs, seed=sum(args))
         ref = oracle.bias_add_nchw_np(oracle.depthwise_nchw_c(x, w, args[6], args[7], args[8]), bias)
         b_, co, p, q = ref.shape
         s, _ = schedule_with_config(key, Config([], None))
-        assert [k.kernel for k in s.specs] == ["depthwise_f32", "bias_add_nchw_f32"]
+        assert [k.kernel for k in s.specs] == ["depthwise_f32"] and s.specs[0].defines["HAS_BIAS"] == 1
         assert rel(run_plan(key, Config([], None), [x, w, bias]), ref) <= TOL
-        gc = {k: [] for k in KEYS}
-        gc["inline"], gc["merge"] = [[1, 0, 0]], [[0, 0, 0]]
-        configs = Config([{k: [] for k in KEYS}, dcfg(b_, co, p, q, 2, 4, 2), {k: [] for k in KEYS}], gc)
-        assert rel(run_plan(key, configs, [x, w, bias]), ref) <= TOL
-        gc["merge"] = [[0, 0, 1]]                  # the depthwise kernel has no bias epilogue
-        with pytest.raises(Exception):
-            schedule_with_config(key, Config(configs.op_config_lst, gc))
+        none = {k: [] for k in KEYS}
+        for merge in (0, 1):
+            # special: nt_store, halo_shfl, lds_planes, lane_items, row_exchange, kernel_fuse
+            variants = [[[0], [0], [0], [1], [0], [1]], [[1], [0], [0], [2], [0], [0]]]
+            if args[4] == 1 and args[6] == 1:
+                variants += [[[0], [1], [0], [1], [0], [1]],      # shuffled halo
+                             [[0], [0], [2], [1], [0], [1]],      # planes staged through LDS
+                             [[1], [0], [0], [1], [2], [1]]]      # row exchange
+            for special in variants:
+                gc = {k: [] for k in KEYS}
+                gc["inline"], gc["merge"], gc["special"] = [[1, 0, 0]], [[0, 0, merge]], special
+                configs = Config([none, dcfg(b_, co, p, q, 2, 4, 2), none], gc)
+                s, _ = schedule_with_config(key, configs)
+                want = ["depthwise_f32"] if merge else ["depthwise_f32", "bias_add_nchw_f32"]
+                assert [k.kernel for k in s.specs] == want
+                assert rel(run_plan(key, configs, [x, w, bias]), ref) <= TOL, (merge, special)
         dev = [torch.from_numpy(a).cuda() for a in (x, w, bias)]
         out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
         run_default_schedule(ops, dev + [out], stream=current_stream())
@@ -487,7 +514,7 @@ def test_depthwise_and_one_channel_groups_with_bias(oracle):
     x, w, bias = seeded_inputs(bufs, seed=sum(args))
     ref = oracle.bias_add_nchw_np(oracle.conv2d_nchw_c(x, w, 1, 1, 1, 6), bias)
     s, _ = schedule_with_config(key, Config([], None))
-    assert [k.kernel for k in s.specs] == ["depthwise_f32", "bias_add_nchw_f32"]
+    assert [k.kernel for k in s.specs] == ["depthwise_f32"]
     assert rel(run_plan(key, Config([], None), [x, w, bias]), ref) <= TOL
 
 
@@ -925,6 +952,11 @@ def test_depthwise_vs_oracle(oracle, args, th, tw, waves):
     ((1, 4, 16, 16, 2, 3, 2, 2, 2), 2, 4, 1),     # stride 2, dilation 2, padding 2: two halo columns on the left
     ((1, 4, 13, 16, 2, 3, 2, 1, 2), 2, 4, 1),     # stride 2, dilation 2, padding 1: output rows are not half rows
     ((1, 3, 9, 11, 4, 3, 2, 1, 1), 2, 2, 1),      # odd plane, two outputs per lane row
+    # a ragged last patch whose last stored column reads the right padding through the vectors
+    ((1, 4, 28, 28, 1, 5, 2, 2, 1), 2, 4, 1),     # 5x5, stride 2, padding 2: 14 output columns
+    ((1, 4, 12, 12, 2, 3, 2, 2, 2), 1, 4, 1),     # 3x3, stride 2, dilation 2, padding 2: 6 output columns
+    ((1, 2, 20, 20, 1, 7, 2, 3, 1), 1, 4, 1),     # 7x7, stride 2, padding 3: 10 output columns
+    ((1, 4, 28, 28, 1, 5, 2, 2, 1), 1, 4, 2),
 ])
 def test_depthwise_kernels_of_a_channel_fused_vs_oracle(oracle, args, th, tw, waves):
     """Several kernels per input channel: a lane loads its input patch once and
@@ -944,7 +976,8 @@ def test_depthwise_kernels_of_a_channel_fused_vs_oracle(oracle, args, th, tw, wa
                 cfgs = conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves),
                                  special=[[0], [shfl], [0], [items], [0], [fuse]])
                 s, _ = schedule_with_config(key, cfgs)
-                assert s.specs[-1].defines.get("MFUSE", 0) == fuse and s.specs[-1].defines["SHFL"] == shfl
+                assert s.specs[-1].defines.get("MFUSE", 0) == (fuse if args[4] > 1 else 0)
+                assert s.specs[-1].defines["SHFL"] == shfl
                 out = run_plan(key, cfgs, [x, w])
                 assert rel(out, ref) <= TOL, (fuse, items, shfl)
     # borders: a constant image must give border sums with missing taps

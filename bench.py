@@ -80,17 +80,41 @@ def measured_traffic(name, plan):
     return rec["hbm_bytes_per_launch"], prov
 
 
-def roofline(name, bound, dtype, ops, nbytes, ms, plan):
+NOMINAL_GHZ = 2.4       # the shader clock the published MFMA peaks assume
+
+
+def roofline(name, bound, dtype, ops, nbytes, ms, plan, clock=None):
+    """``clock``: what Measurer.shader_clock read inside the instrumented build of the same kernel
+    in the same process: the sustained shader clock (the published MFMA peaks assume 2.4 GHz; under
+    load the power limit sets the real one, which differs from box to box) and the median life of a
+    workgroup, which a kernel trace's duration and the per-launch event time both have to exceed."""
     traffic, prov = measured_traffic(name, plan)
     if bound == "hbm":
         achieved = nbytes / (ms * 1e-3) / 1e9
-        return {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBS, "traffic": traffic, "traffic_provenance": prov}
-    peak = PEAK_I8_TOPS if dtype == "i8" else PEAK_F32_TFLOPS
-    achieved = ops / (ms * 1e-3) / 1e12
-    return {"bound": "mfma", "achieved": achieved, "peak": peak,
-            "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak,
-            "traffic": traffic, "traffic_provenance": prov}
+        out = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+               "frac": achieved / PEAK_HBM_GBS, "traffic": traffic, "traffic_provenance": prov}
+    else:
+        peak = PEAK_I8_TOPS if dtype == "i8" else PEAK_F32_TFLOPS
+        achieved = ops / (ms * 1e-3) / 1e12
+        out = {"bound": "mfma", "achieved": achieved, "peak": peak,
+               "unit": "TOP/s" if dtype == "i8" else "TFLOP/s", "frac": achieved / peak,
+               "traffic": traffic, "traffic_provenance": prov}
+    if clock:
+        out["shader_clock_ghz"] = clock["ghz"]
+        out["shader_clock_ghz_p5_p95"] = [clock["ghz_min"], clock["ghz_max"]]
+        out["workgroup_life_ms"] = clock["workgroup_us"] * 1e-3
+        if bound == "mfma":
+            # the same fraction against the peak at the clock the part sustains under this load
+            out["frac_at_sustained_clock"] = out["frac"] * NOMINAL_GHZ / clock["ghz"]
+    return out
+
+
+def shader_clock(m, plan):
+    try:
+        return m.shader_clock(plan, ms=TIMED_WINDOW_MS, warm_ms=WARM_MS)
+    except Exception as e:  # noqa: BLE001 - the clock is an annotation, the timing stands without it
+        print("shader clock probe failed: %s" % e, file=sys.stderr)
+        return None
 
 
 def gpu_workload(key, seed=0):
@@ -273,6 +297,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
+    ap.add_argument("--no-clock", action="store_true",
+                    help="skip the in-kernel shader clock probe (an instrumented build of the same kernel, "
+                         "run after the timing; under a profiler it would show up as extra dispatches)")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="instead of a workload, run a plain device copy of this many MiB "
                          "(bandwidth yardstick; calibrates FETCH_SIZE/WRITE_SIZE)")
@@ -333,7 +360,7 @@ def main():
     if not ok:
         raise RuntimeError("headline plan fails the correctness gate (metric %g)" % metric)
     k_ms, _ = kernel_ms(built, m)
-    roof = roofline(name, bound, dtype, ops, nbytes, k_ms, plan)
+    roof = roofline(name, bound, dtype, ops, nbytes, k_ms, plan, None if args.no_clock else shader_clock(m, plan))
     roof["kernel"] = plan.specs[-1].kernel
     roof["kernel_ms"] = k_ms
     # 24 000 launches of an empty kernel: left out of the short runs that a profiler wraps
@@ -346,7 +373,7 @@ def main():
         for (wname, wkey, wops, wbytes, wbound, wdtype) in WORKLOADS:
             b, mm, pl = gpu_workload(wkey)
             ms, met = kernel_ms(b, mm)
-            r = roofline(wname, wbound, wdtype, wops, wbytes, ms, pl)
+            r = roofline(wname, wbound, wdtype, wops, wbytes, ms, pl, None if args.no_clock else shader_clock(mm, pl))
             entry = {"workload": wname, "ms": ms, "dtype": wdtype,
                      "throughput": wops / (ms * 1e-3) / 1e12,
                      "throughput_unit": "TOP/s" if wdtype == "i8" else "TFLOP/s",

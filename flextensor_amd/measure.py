@@ -224,6 +224,38 @@ class Measurer(object):
         torch.cuda.synchronize()
         return ok, metric
 
+    def shader_clock(self, plan, ms=25.0, warm_ms=150.0):
+        """The shader clock ``plan``'s main kernel sustains, read inside the kernel: the
+        instrumented build of its template (KernelPlan.with_clock_probe) runs back to back for
+        ``warm_ms`` + ``ms`` milliseconds like a timed measurement, and every workgroup of the last
+        launch reports the shader clocks (s_memtime) and the ticks of the constant 100 MHz counter
+        (s_memrealtime) of its life. Returns {"ghz": median ratio, "ghz_min", "ghz_max" (5th and
+        95th percentile over the workgroups), "workgroup_us": median life of a workgroup,
+        "workgroups": how many reported}. The result of the instrumented run is checked too."""
+        import torch
+        probe = plan.with_clock_probe()
+        built = probe.build()
+        try:
+            first = self.sets[0]
+            built(*first)
+            torch.cuda.synchronize()
+            ok, metric = self.check(first[-1])
+            if not ok:
+                raise WrongResult("instrumented build differs from the default schedule (metric %g)" % metric)
+            one = built.time(self.sets, warmup=2, iters=5)
+            built.time(self.sets, warmup=1, iters=max(int(ms / max(one, 1e-4)), 5), warm_ms=warm_ms)
+            torch.cuda.synchronize()
+            clk = built.scratch["clk_probe"].cpu().numpy().astype(np.float64)
+        finally:
+            built.close()
+        clk = clk[clk[:, 1] >= 20]          # workgroups that found no work live a few ticks
+        if len(clk) == 0:
+            return None
+        ghz = clk[:, 0] / clk[:, 1] * 0.1   # clocks per 10 ns
+        return {"ghz": float(np.median(ghz)), "ghz_min": float(np.percentile(ghz, 5)),
+                "ghz_max": float(np.percentile(ghz, 95)), "workgroup_us": float(np.median(clk[:, 1]) / 100.0),
+                "workgroups": int(len(clk))}
+
     def evaluate(self, plan, number=10, warmup=2, warm_ms=WARM_MS, timeout=0.0):
         """ms per run of ``plan``; raises on build failure or wrong output.
         Candidates are compiled between measurements, so each one meets an

@@ -37,8 +37,30 @@ class KernelPlan(object):
     def build(self, static_workspace=False):
         return BuiltPlan(self, static_workspace=static_workspace)
 
+    def with_clock_probe(self):
+        """A copy of the plan whose main kernel is the instrumented build of its template
+        (FT_CLKPROBE): every workgroup writes the shader clocks and the ticks of the 100 MHz
+        counter it lived into the workspace ``clk_probe`` ([workgroups][2] int64). Same work,
+        same launch geometry; used to read the clock the kernel sustains, never timed."""
+        import copy
+        idx = [i for i, s in enumerate(self.specs) if s.template in PROBE_TEMPLATES]
+        if not idx:
+            raise ValueError("no kernel of this plan can carry the clock probe")
+        specs = list(self.specs)
+        spec = copy.copy(specs[idx[-1]])
+        spec.defines = dict(spec.defines, CLKPROBE=1)
+        spec.args = list(spec.args) + [("buf", "clk_probe")]
+        nwg = spec.grid[0] * spec.grid[1] * spec.grid[2]
+        spec.workspace = dict(spec.workspace, clk_probe=((nwg, 2), "int64"))
+        specs[idx[-1]] = spec
+        return KernelPlan(self.task_key, self.bufs, specs, self.intermediates, self.configs)
+
     def __repr__(self):
         return "KernelPlan(%s: %s)" % (self.task_key, ", ".join(s.kernel for s in self.specs))
+
+
+# templates that take the FT_CLKPROBE instrumentation
+PROBE_TEMPLATES = ("igemm_f32.hip", "gemm_i8.hip", "depthwise_f32.hip")
 
 
 _TORCH_DTYPES = None
@@ -48,7 +70,8 @@ def _torch_dtype(name):
     global _TORCH_DTYPES
     import torch
     if _TORCH_DTYPES is None:
-        _TORCH_DTYPES = {"float32": torch.float32, "int8": torch.int8, "int32": torch.int32}
+        _TORCH_DTYPES = {"float32": torch.float32, "int8": torch.int8, "int32": torch.int32,
+                         "int64": torch.int64}
     return _TORCH_DTYPES[name]
 
 
@@ -84,7 +107,7 @@ class BuiltPlan(object):
                 n = 1
                 for d in shape:
                     n *= int(d)
-                nbytes = (n * {"float32": 4, "int32": 4, "int8": 1}[dtype] + 15) // 16 * 16
+                nbytes = (n * {"float32": 4, "int32": 4, "int8": 1, "int64": 8}[dtype] + 15) // 16 * 16
                 self.static_layout[name] = (offset, nbytes, 0 if name.endswith("_parts") else 1)
                 offset = (offset + nbytes + 255) // 256 * 256
             if offset > rt.STATIC_WS_BYTES:

@@ -94,6 +94,22 @@
 #define CP FT_CP
 #define CQ FT_CQ
 
+/* FT_CLKPROBE: an instrumented build that measures the shader clock the kernel runs at. Every
+ * workgroup writes, through one more argument, how many shader clocks (s_memtime) and how many ticks
+ * of the constant 100 MHz counter (s_memrealtime) passed between its first instruction and the
+ * completion of its first wavefront's last store. */
+#ifdef FT_CLKPROBE
+#define CLK_PARAM , unsigned long long* __restrict__ ft_clk
+#define CLK_BEGIN const unsigned long long ft_t0 = __builtin_readcyclecounter(), ft_r0 = wall_clock64();
+#define CLK_END do { __builtin_amdgcn_s_waitcnt(0x0F70); \
+        if (threadIdx.x == 0) { ft_clk[2 * blockIdx.x] = __builtin_readcyclecounter() - ft_t0; \
+                                ft_clk[2 * blockIdx.x + 1] = wall_clock64() - ft_r0; } } while (0)
+#else
+#define CLK_PARAM
+#define CLK_BEGIN
+#define CLK_END do { } while (0)
+#endif
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
@@ -147,8 +163,9 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O BIAS_PARAM)
+                   float* __restrict__ O BIAS_PARAM CLK_PARAM)
 {
+    CLK_BEGIN
     __shared__ __attribute__((aligned(16))) float sx[LDSP * PS];
     __shared__ __attribute__((aligned(16))) float sw[LDSP * 12];     /* 3 taps + 1 pad per kernel row */
     const int tid = threadIdx.x;
@@ -216,6 +233,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
         O4[(size_t)plane * PLANE4 + rem] = acc;
 #endif
     }
+    CLK_END;
 }
 #elif WX > 0
 #if !(STRH == 1 && STRW == 1 && DILH == 1 && DILW == 1 && CR == 3 && CS == 3 && PADH == 1 && PADW == 1 && CP == CH && CQ == CW && CW % 4 == 0 && FACT == 1)
@@ -239,8 +257,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O BIAS_PARAM)
+                   float* __restrict__ O BIAS_PARAM CLK_PARAM)
 {
+    CLK_BEGIN
     /* window chunk ro * Q4 + col of a wavefront holds (row r0 - 1 + ro, chunk col) of its plane.
      * Idle lanes (LPW .. 63) read the chunk their own lane number points at, like the busy ones:
      * 64 consecutive chunks per read, which the LDS serves without a bank conflict (an idle lane
@@ -328,6 +347,7 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #endif
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), ro, (int)vo[i], 0, ST_AUX);
     }
+    CLK_END;
 }
 #else
 /* Every global access of the direct kernel is a raw buffer access: an
@@ -344,8 +364,9 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 
 extern "C" __global__ __launch_bounds__(NT)
 void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
-                   float* __restrict__ O BIAS_PARAM)
+                   float* __restrict__ O BIAS_PARAM CLK_PARAM)
 {
+    CLK_BEGIN
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, X_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(Wt), 0, W_BYTES, 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, O_BYTES, 0x00020000);
@@ -537,5 +558,6 @@ void depthwise_f32(const float* __restrict__ X, const float* __restrict__ Wt,
 #endif
         }
     }
+    CLK_END;
 }
 #endif

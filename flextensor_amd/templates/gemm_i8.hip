@@ -120,8 +120,12 @@ typedef i32x4 acc_t;
 #define OOB 0x80000000u
 #define TILES_M ((M + BM - 1) / BM)
 #define TILES_N ((N + BN - 1) / BN)
-/* KP = K rounded up to a multiple of 64 (host checks KP % BK == 0 and
- * K % 16 == 0); chunks beyond K are zero-filled by the load predicate. */
+/* KP = K rounded up to a multiple of 64 (host checks KP % BK == 0); chunks
+ * beyond K are zero-filled by the load predicate. When K is no multiple of 16
+ * the rows of A and B are not 16-byte aligned and the last chunk of a row is
+ * partly beyond it (those bytes are the next row's, not zeros): the chunk is
+ * then put together from dword loads (K % 4 == 0) or byte loads, each with its
+ * own predicate. Register-staged pipelines only. */
 #define KT (KP / BK)
 
 #if BK % MFMA_K != 0
@@ -137,8 +141,8 @@ typedef i32x4 acc_t;
 #define EA ((A_CHUNKS + NT - 1) / NT)
 #define EB ((B_CHUNKS + NT - 1) / NT)
 #if DTL
-#if PAD > 0 || STAGES != 2 || A_CHUNKS % NT != 0 || B_CHUNKS % NT != 0
-#error "direct-to-LDS tiles need unpadded rows, two buffers and whole rounds of chunks"
+#if PAD > 0 || STAGES != 2 || A_CHUNKS % NT != 0 || B_CHUNKS % NT != 0 || K % 16 != 0
+#error "direct-to-LDS tiles need unpadded rows, two buffers, whole rounds of chunks and K % 16 == 0"
 #endif
 #if DTL == 3 && ((BK / MFMA_K) % 2 != 0 || REP_M * REP_N / 4 + REP_M + REP_N > REP_M * REP_N || REP_M * REP_N / 4 + EA + EB > REP_M * REP_N)
 #error "the pinned schedule needs an even number of k-steps per tile and enough MFMAs per k-step to interleave with"
@@ -146,10 +150,27 @@ typedef i32x4 acc_t;
 typedef __attribute__((address_space(3))) void lds_void;
 #endif
 
+/* FT_CLKPROBE: an instrumented build that measures the shader clock the kernel runs at. Every
+ * workgroup writes, through one more argument, how many shader clocks (s_memtime) and how many ticks
+ * of the constant 100 MHz counter (s_memrealtime) passed between its first instruction and the
+ * completion of its first wavefront's last store. */
+#ifdef FT_CLKPROBE
+#define CLK_PARAM , unsigned long long* __restrict__ ft_clk
+#define CLK_BEGIN const unsigned long long ft_t0 = __builtin_readcyclecounter(), ft_r0 = wall_clock64();
+#define CLK_END do { __builtin_amdgcn_s_waitcnt(0x0F70); \
+        if (threadIdx.x == 0) { ft_clk[2 * blockIdx.x] = __builtin_readcyclecounter() - ft_t0; \
+                                ft_clk[2 * blockIdx.x + 1] = wall_clock64() - ft_r0; } } while (0)
+#else
+#define CLK_PARAM
+#define CLK_BEGIN
+#define CLK_END do { } while (0)
+#endif
+
 extern "C" __global__ __launch_bounds__(NT)
 void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ B,
-             int* __restrict__ C)
+             int* __restrict__ C CLK_PARAM)
 {
+    CLK_BEGIN
     __shared__ __attribute__((aligned(16))) signed char As[STAGES][BM * SROW];
     __shared__ __attribute__((aligned(16))) signed char Bs[STAGES][BN * SROW];
 
@@ -223,19 +244,43 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
 
     i32x4 areg[PD][EA], breg[PD][EB];
 
+    /* the 16 bytes k0 + col .. k0 + col + 15 of the row whose chunk offset is vo */
+    auto load_chunk = [&](__amdgpu_buffer_rsrc_t rsrc, unsigned vo, int k0, int col) -> i32x4 {
+#if K % 16 == 0
+        return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)vo, k0, 0));
+#elif K % 4 == 0
+        i32x4 v;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const unsigned o = (vo != OOB && k0 + col + 4 * d < K) ? vo + 4 * d : OOB;
+            v[d] = (int)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)o, k0, 0);
+        }
+        return v;
+#else
+        i32x4 v = (i32x4)(0);
+#pragma unroll
+        for (int b = 0; b < 16; ++b) {
+            const unsigned o = (vo != OOB && k0 + col + b < K) ? vo + b : OOB;
+            const unsigned byte = (unsigned)__builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)o, k0, 0) & 0xffu;
+            v[b / 4] |= (int)(byte << (8 * (b % 4)));
+        }
+        return v;
+#endif
+    };
+
     auto load_global = [&](int kt, int set) {
         const int k0 = kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
             unsigned vo = a_voff[e];
             if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
-            areg[set][e] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (int)vo, k0, 0));
+            areg[set][e] = load_chunk(rsrc_a, vo, k0, a_col[e]);
         }
 #pragma unroll
         for (int e = 0; e < EB; ++e) {
             unsigned vo = b_voff[e];
             if (KP != K) vo = (k0 + b_col[e] < K) ? vo : OOB;
-            breg[set][e] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)vo, k0, 0));
+            breg[set][e] = load_chunk(rsrc_b, vo, k0, b_col[e]);
         }
     };
 
@@ -602,4 +647,5 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         }
     }
 #endif
+    CLK_END;
 }

@@ -161,7 +161,7 @@ class GemmView(object):
             raise InvalidConfig("operator kind %s has no GEMM view" % kind)
         # K as the kernels iterate it: fp32 pads the tail up to a multiple of
         # 16 (int8: 64) with zero-filling loads unless it already is a multiple
-        # of 8; int8 needs K % 16 == 0.
+        # of 8.
         if min(self.M, self.N, self.K) < 1:
             raise InvalidConfig("empty operator: M, N, K = %d, %d, %d" % (self.M, self.N, self.K))
         if self.dtype == "int8":
@@ -384,8 +384,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         mfma_k = 32 if mfm == 32 else 64
         if bk % mfma_k != 0:
             raise InvalidConfig("BK must be a multiple of the MFMA K extent")
-        if view.K % 16 != 0:
-            raise InvalidConfig("int8 GEMM needs K to be a multiple of 16")
+        if view.K % 16 != 0 and depth >= 6:
+            # rows that are not 16-byte aligned: chunks are put together from dword or byte loads in
+            # registers, which the loads that write LDS directly cannot do
+            raise InvalidConfig("int8 tiles straight into LDS need K to be a multiple of 16")
         pad = int(_special(special, "lds_pad")[0])
         pad = -1 if pad < 0 else pad * 4
         if pad >= 0 and pad % 16 != 0:
@@ -438,8 +440,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     else:
         bv = 1
     dtl = depth >= 5          # fp32: tiles loaded straight into LDS
-    if dtl and view.trans_a:
-        raise InvalidConfig("a transposed A operand is transposed in registers: register-staged pipelines only")
+    if dtl and view.trans_a and (bm % 64 or av != 4):
+        raise InvalidConfig("direct-to-LDS tiles of a transposed A operand need tile rows of a multiple of 64 "
+                            "and M a multiple of 4")
     if dtl:
         if view.mode == 0 and view.N % 4 == 0 and bn % 64 == 0 and (bpad_auto or bpad == 0):
             bv, bpad = 4, 0   # B in 16-byte chunks too: unpadded rows, columns swizzled by k

@@ -241,8 +241,8 @@ typedef f32x4 acc_t;
 
 /* ---- A tile: BM x BK, vectors of AV floats along K (along M when A is stored [K][M]) */
 #if TA
-#if MODE == 1 || DTL
-#error "a transposed A operand: dense GEMM modes, register-staged pipelines"
+#if MODE == 1
+#error "a transposed A operand: dense GEMM modes only"
 #endif
 #define A_CHUNKS_ROW (BM / AV)
 #define A_CHUNKS (BK * A_CHUNKS_ROW)
@@ -316,6 +316,19 @@ typedef f32x4 acc_t;
 #define BSW_R(g) (g)
 #define BSW_C(g) 0
 #endif
+#endif
+#endif
+#if TA
+/* A stored [K][M]: its tile travels like the plain GEMM's B, in 16-byte chunks along M into
+ * unpadded rows [BK][BM], the chunks of row k XOR-ed on the global side so that the lane groups
+ * of an MFMA operand read (rows 4g + s) use different banks; the fragments are read as scalars. */
+#if BM % 64 != 0
+#error "direct-to-LDS tiles of a transposed A need rows of a multiple of 64 floats"
+#endif
+#if MFMA == 16
+#define TSWK(k) ((((k) >> 2) & 3) << 2)
+#else
+#define TSWK(k) ((((k) >> 2) & 1) << 3)
 #endif
 #endif
 typedef __attribute__((address_space(3))) void lds_void;
@@ -417,6 +430,22 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 #define RED_FLOATS ((WAVES_K - 1) * NT * REP_M * REP_N * NACC)
 #define SMEM_FLOATS (TILE_FLOATS > RED_FLOATS ? TILE_FLOATS : RED_FLOATS)
 
+/* FT_CLKPROBE: an instrumented build that measures the shader clock the kernel runs at. Every
+ * workgroup writes, through one more argument, how many shader clocks (s_memtime) and how many ticks
+ * of the constant 100 MHz counter (s_memrealtime) passed between its first instruction and the
+ * completion of its first wavefront's last store. */
+#ifdef FT_CLKPROBE
+#define CLK_PARAM , unsigned long long* __restrict__ ft_clk
+#define CLK_BEGIN const unsigned long long ft_t0 = __builtin_readcyclecounter(), ft_r0 = wall_clock64();
+#define CLK_END do { __builtin_amdgcn_s_waitcnt(0x0F70); \
+        if (threadIdx.x == 0) { ft_clk[2 * blockIdx.x] = __builtin_readcyclecounter() - ft_t0; \
+                                ft_clk[2 * blockIdx.x + 1] = wall_clock64() - ft_r0; } } while (0)
+#else
+#define CLK_PARAM
+#define CLK_BEGIN
+#define CLK_END do { } while (0)
+#endif
+
 extern "C" __global__ __launch_bounds__(NTW)
 void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
                float* __restrict__ C
@@ -426,8 +455,9 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #if HAS_BIAS
                , const float* __restrict__ bias
 #endif
-               )
+               CLK_PARAM)
 {
+    CLK_BEGIN
     __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
     /* k-group of this wavefront (NT is a multiple of 64, so it is uniform
      * over a wavefront; readfirstlane tells the compiler so) */
@@ -455,7 +485,9 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     for (int e = 0; e < EA; ++e) {
         const int q = tid + e * NT;
         a_row[e] = q / A_CHUNKS_ROW;
-#if DTL
+#if DTL && TA
+        a_col[e] = ((q % A_CHUNKS_ROW) ^ TSWK(a_row[e])) * AV;      /* a_row is k, a_col the first of four rows m */
+#elif DTL
         /* chunk q lands at float 4*q of the tile, i.e. at physical chunk
          * q % A_CHUNKS_ROW of its row: fetch the logical chunk that belongs there */
         a_col[e] = ACOL(a_row[e], (q % A_CHUNKS_ROW) * AV);
@@ -683,9 +715,15 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         for (int e = 0; e < EA; ++e) {
             if (e % nparts != part) continue;
             unsigned vo = a_voff[e];
+#if TA
+            if (KP != K) vo = (k0 + a_row[e] < K) ? vo : OOB;
+            if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))
+                dma16(desc_a, &As[buf][(e * NT + wv * 64) * 4], vo, k0 * (M * 4));
+#else
             if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
             if ((A_CHUNKS % NT == 0) || (e * NT + wv * 64 < A_CHUNKS))     /* whole wavefronts only */
                 dma16(desc_a, &As[buf][(e * NT + wv * 64) * 4], vo, k0 * 4);
+#endif
         }
     };
     auto dma_b_one = [&](int kt, int buf, int e) {
@@ -890,6 +928,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 
     /* ---- MFMA operands: LDS -> registers -> matrix core ------------------ */
     /* lane constants of the fragment reads (the same for every tile and buffer) */
+#if TA && DTL
+    /* physical column of row m in tile row kb + 4*lg + s (see TSWK): m ^ (lane group part) */
+    int acolx[REP_M];
+#pragma unroll
+    for (int i = 0; i < REP_M; ++i)
+        acolx[i] = (wm * REP_M * MFMA + i * MFMA + li) ^ (MFMA == 16 ? (lg << 4) : (lg << 5));
+#endif
     const int arow = wm * REP_M * MFMA + li;   /* + i*MFMA: SWZ is the same when MFMA % 16 == 0 */
     int acls[SWZ_CLASSES];
 #pragma unroll
@@ -920,10 +965,19 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     /* the operands of the k block [kb, kb + KBLK) of the tile in LDS buffer buf:
      * a[i] = four k values of row block i, b[s][j] = k value s of column block j */
     auto read_block = [&](int buf, int kb, f32x4 (&a)[REP_M], float (&b)[4][REP_N]) {
+#if TA && DTL
+        const float* at = &As[buf][(4 * lg) * BM];
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                a[i][s] = at[(kb + s) * BM + acolx[i]];
+#else
         const float* as = &As[buf][arow * SA];
 #pragma unroll
         for (int i = 0; i < REP_M; ++i)
             a[i] = *reinterpret_cast<const f32x4*>(as + i * MFMA * SA + SWZ_HI(kb) + acls[SWZ_CLS(kb)]);
+#endif
 #if MODE == 2
         const float* bs = &Bs[buf][brow * SB];
 #pragma unroll
@@ -1202,4 +1256,5 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         }
     }
 #endif
+    CLK_END;
 }

@@ -25,7 +25,7 @@ from flextensor_amd.task import (TASK_TABLE, Task, register, gemm, gemm_int8, co
                                  depthwise_conv2d)
 from flextensor_amd.nn import gemm as op_gemm  # noqa: E402
 from flextensor_amd.te import placeholder  # noqa: E402
-from flextensor_amd.templates.gfx950 import special_knobs  # noqa: E402
+from flextensor_amd.templates.gfx950 import InvalidConfig, special_knobs  # noqa: E402
 from flextensor_amd.utils import Config, ceil_div  # noqa: E402
 
 TOL = 1e-5
@@ -697,8 +697,15 @@ def test_gemm_transpose_a_vs_oracle(oracle):
         for cfg in cfgs:
             out = run_plan(key, Config([cfg] if cfg else [], None), [a, b])
             assert rel(out, ref) <= TOL, (M, K, N, tb, cfg)
-        with pytest.raises(Exception):      # tiles straight into LDS cannot transpose
+        with pytest.raises(Exception):      # tiles straight into LDS: a transposed A needs tile rows of 64 floats
             schedule_with_config(key, Config([gcfg(M, N, kp, 2, 1, 2, 1, 16, 16, st=5)], None))
+        if M % 4 == 0:
+            # tiles straight into LDS: the [K][M] tile lands as it lies in memory, fragments read as scalars
+            dtl = [gcfg(M, N, kp, 4, 1, 2, 1, 16, 16, st=5), gcfg(M, N, kp, 2, 1, 1, 2, 32, 32, st=8),
+                   gcfg(M, N, kp, 2, 2, 2, 1, 16, 32, st=6), gcfg(M, N, kp, 4, 1, 4, 1, 16, 32, st=8)]
+            for cfg in dtl:
+                out = run_plan(key, Config([cfg], None), [a, b])       # default LDS layout: swizzled, unpadded rows
+                assert rel(out, ref) <= TOL, (M, K, N, tb, cfg)
         # and the default-schedule kernel the search checks candidates against
         dev = [torch.from_numpy(x).cuda() for x in (a, b)]
         out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
@@ -743,6 +750,27 @@ def test_gemm_int8_row_vector_stores(oracle, M, K, N, kn, store):
     """nt_store bit 1: the MFMA computes the transposed tile so that a lane
     holds four consecutive columns of one row."""
     _gemm_int8_case(oracle, M, K, N, kn, store)
+
+
+@pytest.mark.parametrize("M,K,N,kn", [
+    (136, 200, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64)),              # K % 16 = 8: rows 8-byte aligned, dword loads
+    (96, 100, 80, dict(wm=1, rm=2, wn=1, rn=1, mf=16, bk=64, st=1)),         # K % 16 = 4: a 4-byte tail
+    (64, 67, 48, dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=64, st=3)),          # odd K: byte loads, one tile
+    (80, 333, 96, dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=128, st=5)),        # odd K, three tiles, fragment prefetch
+    (48, 18, 40, dict(wm=1, rm=1, wn=1, rn=1, mf=16, bk=64)),                # K below one MFMA step
+])
+def test_gemm_int8_k_not_a_multiple_of_16(oracle, M, K, N, kn):
+    """The operator is defined for any reduce length (legacy/gemm_int8.py:15-21): rows that are not
+    16-byte aligned are loaded in dwords or bytes, the bytes of the last chunk beyond the row (they
+    belong to the next row) are replaced by zeros. Tiles straight into LDS refuse such a K."""
+    _gemm_int8_case(oracle, M, K, N, kn, None)
+    a = np.full((M, K), -128, np.int8)
+    b = np.full((N, K), -128, np.int8)
+    key = key_of("gemm", "gemm_int8", (M, K, N))
+    out = run_plan(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], None), [a, b])
+    assert np.array_equal(out, np.full((M, N), K * 16384, np.int32))          # every tail byte counted once
+    with pytest.raises(Exception):
+        schedule_with_config(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **dict(kn, st=6))], None))
 
 
 def _gemm_int8_case(oracle, M, K, N, kn, store):
@@ -975,6 +1003,10 @@ def test_depthwise_kernels_of_a_channel_fused_vs_oracle(oracle, args, th, tw, wa
             for shfl in shuffles:
                 cfgs = conv_cfgs(dcfg(b_, co, p, q, min(th, p), min(tw, q), waves),
                                  special=[[0], [shfl], [0], [items], [0], [fuse]])
+                if items == 2 and args[5] >= 7:
+                    with pytest.raises(InvalidConfig):      # two 7x7 patches per lane do not fit the registers
+                        schedule_with_config(key, cfgs)
+                    continue
                 s, _ = schedule_with_config(key, cfgs)
                 assert s.specs[-1].defines.get("MFUSE", 0) == (fuse if args[4] > 1 else 0)
                 assert s.specs[-1].defines["SHFL"] == shfl

@@ -698,15 +698,32 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     };
     const i32x4 desc_a = descriptor(A, (unsigned)A_BYTES);
     const i32x4 desc_b = descriptor(B, (unsigned)B_BYTES);
+    /* The descriptor, the LDS address and the scalar offset are wave-uniform by construction.
+     * With more than two buffers inside the K-streaming segment loop (a buffer index carried around
+     * a loop that has lane-dependent exits) the compiler no longer sees that and would hand the
+     * instruction vector registers, so there it is told; everywhere else it knows, and telling it
+     * anyway costs instructions in the main loop. */
+#if SK_PER > 0 && STAGES > 2
+#define DMA_UNIFORM(x) __builtin_amdgcn_readfirstlane((int)(x))
+    auto uniform4 = [](const i32x4& v) {
+        i32x4 r;
+        r[0] = __builtin_amdgcn_readfirstlane(v[0]); r[1] = __builtin_amdgcn_readfirstlane(v[1]);
+        r[2] = __builtin_amdgcn_readfirstlane(v[2]); r[3] = __builtin_amdgcn_readfirstlane(v[3]);
+        return r;
+    };
+#else
+#define DMA_UNIFORM(x) (x)
+    auto uniform4 = [](const i32x4& v) -> const i32x4& { return v; };
+#endif
     auto dma16 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
-        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        const unsigned lds_addr = (unsigned)DMA_UNIFORM((unsigned)(__UINTPTR_TYPE__)(lds_void*)dst);
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
+                     :: "s"(lds_addr), "v"(vo), "s"(uniform4(rsrc)), "s"(DMA_UNIFORM(so)) : "memory", "m0");
     };
     auto dma4 = [&](const i32x4& rsrc, const float* dst, unsigned vo, int so) {
-        const unsigned lds_addr = (unsigned)(__UINTPTR_TYPE__)(lds_void*)dst;
+        const unsigned lds_addr = (unsigned)DMA_UNIFORM((unsigned)(__UINTPTR_TYPE__)(lds_void*)dst);
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-                     :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
+                     :: "s"(lds_addr), "v"(vo), "s"(uniform4(rsrc)), "s"(DMA_UNIFORM(so)) : "memory", "m0");
     };
     /* part p of np: the loads e of the tile with e mod np == p (A first, then B) */
     auto dma_tile_a = [&](int kt, int buf, int part = 0, int nparts = 1) {

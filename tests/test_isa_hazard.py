@@ -205,3 +205,15 @@ def test_depthwise_lane_shifts_run_with_every_lane_switched_on(special):
     text = isa_hazards.assembly_of(plan.specs[-1])
     assert "_dpp" in text, "the kernel is expected to shift lanes with DPP"
     assert isa_hazards.check_plan(plan) == []
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+@pytest.mark.parametrize("shape_index", [0, 3, 4, 7, 8, 11, 13, 14, 18, 20])
+def test_random_points_of_the_spaces_pass_the_static_checks(shape_index):
+    """The generated assembly of points drawn at random from the schedule spaces (the same points
+    the device parity test runs): no accumulator read before the matrix core has written it, no
+    arrival counted ahead of the slot stores, no lane shift under a narrowed exec mask."""
+    from random_points import point
+    for number in (0, 4):
+        kind, key, args, configs, plan = point(shape_index, number)
+        assert isa_hazards.check_plan(plan) == [], (key, configs)

@@ -38,6 +38,12 @@
 //               (left to itself the compiler issues the fragment reads right
 //               before their first use and waits for them)
 //   NT_STORE    1: non-temporal stores for C
+//   EARLYST     1 (with DTL 2 and two k-steps per tile): the last tile is multiplied
+//               block by block instead of k-step by k-step, and every accumulator
+//               block is stored as soon as its last MFMA has been issued and the
+//               next group's MFMAs cover the distance to the read: the stores of C
+//               start a tile's time before the workgroup's last MFMA instead of
+//               behind it
 //   CVEC        1: the MFMA operands are swapped (the core computes the
 //               transposed tile), so a lane holds four consecutive columns of
 //               one row of C and writes them with one 128-bit store
@@ -76,6 +82,11 @@
 #define CVEC FT_CVEC
 #else
 #define CVEC 0
+#endif
+#ifdef FT_EARLYST
+#define EARLYST FT_EARLYST
+#else
+#define EARLYST 0
 #endif
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -302,6 +313,58 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         for (int j = 0; j < REP_N; ++j)
             acc[i][j] = (acc_t)(0);
 
+    /* accumulator block (i, j) -> C */
+    auto store_block = [&](int i, int j) {
+#if CVEC
+        /* swapped operands: lane (li, lg) holds C[m = li][n = 4*lg + 0..3] (16x16),
+         * or C[m = li][n = 8*q + 4*lg + 0..3] in registers 4q..4q+3 (32x32) */
+        const int m = m0 + (wm * REP_M + i) * MFMA + li;
+#pragma unroll
+        for (int q = 0; q < NACC / 4; ++q) {
+#if MFMA == 32
+            const int n = n0 + (wn * REP_N + j) * MFMA + 8 * q + 4 * lg;
+#else
+            const int n = n0 + (wn * REP_N + j) * MFMA + 4 * lg;
+#endif
+            bool ok = true;
+            if (M % BM != 0) ok = ok && (m < M);
+            if (N % BN != 0) ok = ok && (n < N);      /* N % 4 == 0: whole vectors */
+            if (ok) {
+                i32x4 v4;
+                v4[0] = acc[i][j][4 * q + 0]; v4[1] = acc[i][j][4 * q + 1];
+                v4[2] = acc[i][j][4 * q + 2]; v4[3] = acc[i][j][4 * q + 3];
+                i32x4* dst = reinterpret_cast<i32x4*>(C + (size_t)m * N + n);
+#if NT_STORE
+                __builtin_nontemporal_store(v4, dst);
+#else
+                *dst = v4;
+#endif
+            }
+        }
+#else
+        const int n = n0 + (wn * REP_N + j) * MFMA + li;
+#pragma unroll
+        for (int v = 0; v < NACC; ++v) {
+#if MFMA == 32
+            const int row = 8 * (v / 4) + 4 * lg + (v % 4);
+#else
+            const int row = 4 * lg + v;
+#endif
+            const int m = m0 + (wm * REP_M + i) * MFMA + row;
+            bool ok = true;
+            if (M % BM != 0) ok = ok && (m < M);
+            if (N % BN != 0) ok = ok && (n < N);
+            if (ok) {
+#if NT_STORE
+                __builtin_nontemporal_store(acc[i][j][v], C + (size_t)m * N + n);
+#else
+                C[(size_t)m * N + n] = acc[i][j][v];
+#endif
+            }
+        }
+#endif
+    };
+
     auto compute = [&](int buf) {
         const int arow = wm * REP_M * MFMA + li;
         const int brow = wn * REP_N * MFMA + li;
@@ -464,7 +527,15 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
         };
         i32x4 fa[REP_M], fb[REP_N];
         load_frags(0, 0, fa, fb);
-        for (int kt = 0; kt < KT; ++kt) {
+#if EARLYST
+#if BK != 2 * MFMA_K
+#error "early stores: two k-steps per tile"
+#endif
+#define KT_LOOP (KT - 1)
+#else
+#define KT_LOOP KT
+#endif
+        for (int kt = 0; kt < KT_LOOP; ++kt) {
             const int cur = kt & 1;
             if (kt + 1 < KT) dma_tile(kt + 1, cur ^ 1);
 #pragma unroll
@@ -491,6 +562,36 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
                 }
             }
         }
+#if EARLYST
+        {
+            /* the last tile, block-major: fa/fb hold the fragments of its first k-step, na/nb get
+             * those of its second; blocks go in groups of EG, and the stores of a group are issued
+             * behind the MFMAs of the next group, which cover the distance from an MFMA to the
+             * read of its result */
+            i32x4 na[REP_M], nb[REP_N];
+            load_frags((KT - 1) & 1, MFMA_K, na, nb);
+#define EG 4
+#define NBLK (REP_M * REP_N)
+#pragma unroll
+            for (int g = 0; g <= (NBLK + EG - 1) / EG; ++g) {
+                if (g * EG < NBLK) {
+#pragma unroll
+                    for (int b = g * EG; b < g * EG + EG && b < NBLK; ++b)
+                        acc[b / REP_N][b % REP_N] = MFMA_OP(fa[b / REP_N], fb[b % REP_N], acc[b / REP_N][b % REP_N]);
+#pragma unroll
+                    for (int b = g * EG; b < g * EG + EG && b < NBLK; ++b)
+                        acc[b / REP_N][b % REP_N] = MFMA_OP(na[b / REP_N], nb[b % REP_N], acc[b / REP_N][b % REP_N]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (g > 0) {
+#pragma unroll
+                    for (int b = (g - 1) * EG; b < g * EG && b < NBLK; ++b)
+                        store_block(b / REP_N, b % REP_N);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#endif
 #else
         for (int kt = 0; kt < KT; ++kt) {
             const int cur = kt & 1;
@@ -587,65 +688,12 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
-#if CVEC
-    /* swapped operands: lane (li, lg) holds C[m = li][n = 4*lg + 0..3] (16x16),
-     * or C[m = li][n = 8*q + 4*lg + 0..3] in registers 4q..4q+3 (32x32) */
+#if !EARLYST
 #pragma unroll
-    for (int i = 0; i < REP_M; ++i) {
-        const int m = m0 + (wm * REP_M + i) * MFMA + li;
+    for (int i = 0; i < REP_M; ++i)
 #pragma unroll
-        for (int j = 0; j < REP_N; ++j) {
-#pragma unroll
-            for (int q = 0; q < NACC / 4; ++q) {
-#if MFMA == 32
-                const int n = n0 + (wn * REP_N + j) * MFMA + 8 * q + 4 * lg;
-#else
-                const int n = n0 + (wn * REP_N + j) * MFMA + 4 * lg;
-#endif
-                bool ok = true;
-                if (M % BM != 0) ok = ok && (m < M);
-                if (N % BN != 0) ok = ok && (n < N);      /* N % 4 == 0: whole vectors */
-                if (ok) {
-                    i32x4 v4;
-                    v4[0] = acc[i][j][4 * q + 0]; v4[1] = acc[i][j][4 * q + 1];
-                    v4[2] = acc[i][j][4 * q + 2]; v4[3] = acc[i][j][4 * q + 3];
-                    i32x4* dst = reinterpret_cast<i32x4*>(C + (size_t)m * N + n);
-#if NT_STORE
-                    __builtin_nontemporal_store(v4, dst);
-#else
-                    *dst = v4;
-#endif
-                }
-            }
-        }
-    }
-#else
-#pragma unroll
-    for (int i = 0; i < REP_M; ++i) {
-#pragma unroll
-        for (int j = 0; j < REP_N; ++j) {
-            const int n = n0 + (wn * REP_N + j) * MFMA + li;
-#pragma unroll
-            for (int v = 0; v < NACC; ++v) {
-#if MFMA == 32
-                const int row = 8 * (v / 4) + 4 * lg + (v % 4);
-#else
-                const int row = 4 * lg + v;
-#endif
-                const int m = m0 + (wm * REP_M + i) * MFMA + row;
-                bool ok = true;
-                if (M % BM != 0) ok = ok && (m < M);
-                if (N % BN != 0) ok = ok && (n < N);
-                if (ok) {
-#if NT_STORE
-                    __builtin_nontemporal_store(acc[i][j][v], C + (size_t)m * N + n);
-#else
-                    C[(size_t)m * N + n] = acc[i][j][v];
-#endif
-                }
-            }
-        }
-    }
+        for (int j = 0; j < REP_N; ++j)
+            store_block(i, j);
 #endif
     CLK_END;
 }

@@ -294,7 +294,8 @@ def special_knobs(kind):
     if kind in ("gemm", "conv2d_nchw", "batch_gemm", "col_gemm"):
         return {"lds_pad": [[-1, -1], [4, -1], [4, 8], [4, 4], [0, 0], [8, -1], [-1, 0]]}
     if kind == "gemm_int8":
-        return {"lds_pad": [[-1, 0], [4, 0], [0, 0], [8, 0]], "nt_store": [[0], [1], [2], [3]]}
+        return {"lds_pad": [[-1, 0], [4, 0], [0, 0], [8, 0]],
+                "nt_store": [[0], [1], [2], [3], [4], [5], [6], [7]]}
     if kind == "depthwise_conv2d_nchw":
         return {"nt_store": [[0], [1], [2], [3]], "halo_shfl": [[0], [1]], "lds_planes": [[0], [1], [2], [4], [8]],
                 "lane_items": [[1], [2], [3], [4], [6], [8]], "row_exchange": [[0], [1], [2], [3], [4]],
@@ -407,15 +408,20 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         lds = stages * (bm + bn) * (bk + max(pad, 0))
         if lds > LDS_BYTES:
             raise InvalidConfig("LDS tile needs %d bytes" % lds)
-        # nt_store: bit 0 = non-temporal stores, bit 1 = transposed MFMA so that lanes store 128-bit rows
+        # nt_store: bit 0 = non-temporal stores, bit 1 = transposed MFMA so that lanes store 128-bit rows,
+        # bit 2 = the last tile multiplied block by block, every block stored as soon as it is complete
         store_mode = int(_special(special, "nt_store")[0])
         if store_mode & 2 and view.N % 4 != 0:
             raise InvalidConfig("128-bit C stores need N to be a multiple of 4")
+        if store_mode & 4 and (depth != 7 or bk != 2 * mfma_k or kp // bk < 2):
+            raise InvalidConfig("early stores come with pipeline depth 7, two k-steps per tile, two tiles or more")
         D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0, NT_STORE=store_mode & 1)
         if depth >= 6:
             D.update(DTL=depth - 5)
         if store_mode & 2:
             D.update(CVEC=1)
+        if store_mode & 4:
+            D.update(EARLYST=1)
         grid = (gm * gn, 1, 1)
         spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
                           [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])

@@ -285,6 +285,34 @@ def test_k_streaming_plan_is_reusable_and_deterministic(oracle):
         TASK_TABLE[key].special_space.pop("sk_fenced", None)
 
 
+def test_grid_level_split_k_repeats_within_a_few_ulp(oracle):
+    """K parts that meet in C through float atomics (after a zero fill) add in the order the
+    workgroups happen to arrive, so the last bits move from run to run. The bound: every run within
+    1e-5 of the oracle like any other plan, and any two runs within 2e-6 of max|ref| of each other
+    (16 partial sums of magnitude <= max|ref| each, a few ulp of reordering); K streaming and the
+    in-workgroup split, which add in a fixed order, repeat exactly."""
+    M, K, N = 256, 4096, 192
+    register(gemm, "gemm", "gemm", (M, K, N), "rocm", 0)
+    key = key_of("gemm", "gemm", (M, K, N))
+    _, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=12)
+    ref = oracle.gemm_np(a, b)
+    scale = float(np.max(np.abs(ref)))
+    for kn, exact in ((dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, sk=16), False),
+                      (dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=32, sk=4, wk=1), True),
+                      (dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, ks=1, st=3), True)):
+        s, _ = schedule_with_config(key, Config([gcfg(M, N, K, **kn)], None))
+        assert (s.specs[0].kernel == "fill_zero_f32") == (not exact)
+        outs = [run_plan(key, Config([gcfg(M, N, K, **kn)], None), [a, b]) for _ in range(6)]
+        for o in outs:
+            assert rel(o, ref) <= TOL
+        spread = max(float(np.max(np.abs(o.astype(np.float64) - outs[0]))) for o in outs[1:]) / scale
+        if exact:
+            assert spread == 0.0, kn
+        else:
+            assert spread <= 2e-6, spread
+
+
 @pytest.mark.parametrize("M,K,N,kn,pad", [
     (256, 256, 256, dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=32, st=5), [-1, -1]),            # swizzled A rows
     (256, 512, 256, dict(wm=4, rm=1, wn=4, rn=1, mf=16, bk=64, st=5), [-1, 4]),
@@ -745,10 +773,16 @@ def test_gemm_int8_vs_oracle(oracle, M, K, N, kn):
     (200, 320, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, st=5), 2),
     (256, 512, 384, dict(wm=1, rm=4, wn=2, rn=2, mf=16, bk=128), 3),         # same, non-temporal
     (512, 256, 512, dict(wm=2, rm=4, wn=2, rn=4, mf=32, bk=128, gm=2), 3),
+    # bit 2: the last tile block by block, every block stored as soon as it is complete
+    (512, 512, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=64, st=7), 4),        # eight tiles, 32x32x32
+    (200, 336, 136, dict(wm=2, rm=2, wn=1, rn=4, mf=16, bk=128, st=7), 4),       # ragged M and N, K tail, three tiles
+    (256, 256, 256, dict(wm=2, rm=4, wn=2, rn=4, mf=16, bk=128, st=7), 6),       # with 128-bit row stores, two tiles
+    (200, 336, 136, dict(wm=1, rm=3, wn=2, rn=1, mf=16, bk=128, st=7), 7),       # three blocks per wavefront: a ragged last group
+    (512, 1024, 512, dict(wm=4, rm=4, wn=2, rn=8, mf=16, bk=128, st=7), 4),      # the benchmark's tile
 ])
 def test_gemm_int8_row_vector_stores(oracle, M, K, N, kn, store):
     """nt_store bit 1: the MFMA computes the transposed tile so that a lane
-    holds four consecutive columns of one row."""
+    holds four consecutive columns of one row; bit 2: early stores in the last tile."""
     _gemm_int8_case(oracle, M, K, N, kn, store)
 
 

@@ -154,6 +154,51 @@ def build_and_eval_wrapper(lib, task_key, config, op_pos=None, rpc_info=None, re
     return build_and_eval(lib, s, bufs, task.target, task.dev_id, rpc_info, number)
 
 
+class _Plateau(object):
+    """The searches' stopping rule: the best value has moved by less than 2 % for ``patience``
+    looks in a row."""
+
+    def __init__(self, value, patience):
+        self.value, self.patience, self.count = value, patience, 0
+
+    def stalled(self, value):
+        if self.value < float("inf") and math.fabs(value - self.value) < 0.02 * self.value:
+            self.count += 1
+        else:
+            self.value, self.count = value, 0
+        return self.count >= self.patience
+
+
+class _Shelf(object):
+    """Points taken off a WalkerGroup's heap (local minima the walk should leave): the best of
+    them is kept apart from the rest, as the reference's ``minimal`` / ``retired_indices`` pair."""
+
+    def __init__(self):
+        self.best, self.best_value, self.rest = {}, float("inf"), []
+
+    def put(self, indices, value):
+        if value < self.best_value:
+            if self.best_value < float("inf"):
+                self.rest.append((self.best, self.best_value))
+            self.best, self.best_value = indices, value
+        else:
+            self.rest.append((indices, value))
+
+    def best_with(self, group):
+        """(indices, value) of the better of the heap's top and the shelf's best."""
+        if group.top1_value() < self.best_value:
+            return group.top1(), group.top1_value()
+        return self.best, self.best_value
+
+    def pour_into(self, group):
+        """Everything goes back on the heap; the shelf is empty afterwards."""
+        if self.best_value < float("inf"):
+            group.record(self.best, self.best_value, random_reject=False)
+        for indices, value in self.rest:
+            group.record(indices, value, random_reject=False)
+        self.__init__()
+
+
 class Scheduler(object):
     def __init__(self, name, task_key, space, parallel=2, timeout=4.0, trial=100, number=1,
                  early_stop=30, rpc_info=None, rewrite=False, evaluator=None):
@@ -356,8 +401,7 @@ class Scheduler(object):
         best = self.walker_group.top1()
         best_value = self.walker_group.top1_value()
         retired_indices = []
-        value_early_stop = best_value
-        early_stop_count = 0
+        plateau = _Plateau(best_value, self.early_stop)
         cur_lst = self.walker_group.topk(self.parallel, modify=True, with_value=True)
         part = math.ceil(self.trial / 5)
         for trial in range(self.trial):
@@ -382,14 +426,8 @@ class Scheduler(object):
                 if value < best_value:
                     best, best_value = indices, value
             self._log("No. %d | [%.6f] The best currently %.6f" % (trial, time.time(), best_value), best)
-            if value_early_stop < float("inf") and \
-                    math.fabs(best_value - value_early_stop) < 0.02 * value_early_stop:
-                early_stop_count += 1
-            else:
-                value_early_stop = best_value
-                early_stop_count = 0
-            if early_stop_count >= self.early_stop:
-                self._log("Early stop with value %f repeats %d times" % (value_early_stop, early_stop_count))
+            if plateau.stalled(best_value):
+                self._log("Early stop with value %f repeats %d times" % (plateau.value, plateau.count))
                 break
             retired_indices.extend(cur_lst)
             if not self.walker_group.has_more():
@@ -430,102 +468,67 @@ class Scheduler(object):
 
     # ---- neighbourhood search -----------------------------------------
     def _searching_schedule(self, configs, type_keys, use_model=False):
+        """The reference's walk (flextensor/scheduler.py:321-442): start from a good point chosen
+        at random, measure all its neighbours, take a point that none of them beats off the heap,
+        re-measure the leaders every trial/20 trials, one random warm-up batch per trial; stop on
+        a plateau of the best value or when no point has unvisited neighbours left."""
+        group = self.walker_group
         if use_model:
-            self.walker_group.load_or_create_model()
+            group.load_or_create_model()
         self._seed(configs, type_keys)
-        self._warm_up(self.warm_up_epoch, self.warm_up_number, configs, type_keys,
-                      use_model=use_model)
+        self._warm_up(self.warm_up_epoch, self.warm_up_number, configs, type_keys, use_model=use_model)
 
-        minimal = [{}, float("inf")]
-        retired_indices = []
-
-        part = math.ceil(self.trial / 20)
-        value_early_stop = self.walker_group.top1_value()
-        early_stop_count = 0
-        count_incessant_empty_trial = 0
+        shelf = _Shelf()                       # local minima, off the heap so the walk leaves them
+        plateau = _Plateau(group.top1_value(), self.early_stop)
+        remeasure_every = math.ceil(self.trial / 20)
+        barren = 0                             # trials in a row whose start point had no new neighbour
         for trial in range(self.trial):
-            if not self.walker_group.has_more():
+            if not group.has_more():
                 self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
                 continue
-            from_indices, from_value = self.walker_group.top_random(with_value=True)
-            next_indices_lst, action_lst = self.walker_group.full_walk(from_indices, no_repeat=True)
-            next_configs = [self.walker_group.to_config(indices) for indices in next_indices_lst]
-            if len(next_configs) < 1:
-                count_incessant_empty_trial += 1
-            else:
-                count_incessant_empty_trial = 0
-            results = self._cost(configs, next_indices_lst, use_model)
-            self._log("tune [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
-            rewards = [np.tanh(max(from_value - result, 0.0)) for result in results]
-
-            is_local_minimal = True
-            for indices, action, reward, result in zip(next_indices_lst, action_lst, rewards, results):
-                self.walker_group.add_data(action[0], from_indices, action[1], indices, reward)
-                self.walker_group.record(indices, result, random_reject=True)
-                if result < self.walker_group.top1_value():
-                    is_local_minimal = False
-            if is_local_minimal or count_incessant_empty_trial > 0:
-                top = self.walker_group.pop_top()
-                if top.value < minimal[1]:
-                    if minimal[1] < float("inf"):
-                        retired_indices.append(minimal)
-                    minimal = [top.indices, top.value]
-                else:
-                    retired_indices.append([top.indices, top.value])
-            if self.walker_group.top1_value() < minimal[1]:
-                cur_best_value = self.walker_group.top1_value()
-                cur_best = self.walker_group.top1()
-            else:
-                cur_best_value = minimal[1]
-                cur_best = minimal[0]
-            self._log("No. %d | [%.6f] The best currently %.6f" % (trial, time.time(), cur_best_value),
-                      cur_best)
-            if count_incessant_empty_trial >= self.early_stop:
-                self._log("Early stop after continuous no trials %d times" % count_incessant_empty_trial)
+            start, start_value = group.top_random(with_value=True)
+            neighbours, moves = group.full_walk(start, no_repeat=True)
+            barren = barren + 1 if not neighbours else 0
+            costs = self._cost(configs, neighbours, use_model)
+            self._log("tune [%.6f] [ %s]" % (time.time(), "".join("%.6f " % c for c in costs)))
+            beaten = False
+            for point, (name, direction), cost in zip(neighbours, moves, costs):
+                reward = np.tanh(max(start_value - cost, 0.0))
+                group.add_data(name, start, direction, point, reward)
+                group.record(point, cost, random_reject=True)
+                beaten = beaten or cost < group.top1_value()
+            if not beaten or barren:
+                top = group.pop_top()
+                shelf.put(top.indices, top.value)
+            leader, leader_value = shelf.best_with(group)
+            self._log("No. %d | [%.6f] The best currently %.6f" % (trial, time.time(), leader_value), leader)
+            if barren >= self.early_stop:
+                self._log("Early stop after continuous no trials %d times" % barren)
                 break
             # "no progress" = the best moved by less than 2 % (the reference uses
             # an absolute 0.02 ms, which every microsecond-scale kernel satisfies)
-            if value_early_stop < float("inf") and \
-                    math.fabs(cur_best_value - value_early_stop) < 0.02 * value_early_stop:
-                early_stop_count += 1
-            else:
-                value_early_stop = cur_best_value
-                early_stop_count = 0
-            if early_stop_count >= self.early_stop:
-                self._log("Early stop with value %f repeats %d times" % (value_early_stop, early_stop_count))
+            if plateau.stalled(leader_value):
+                self._log("Early stop with value %f repeats %d times" % (plateau.value, plateau.count))
                 break
-            if (trial + 1) % part == 0:
-                # re-measure the current top points one after another
-                if minimal[1] < float("inf"):
-                    self.walker_group.record(minimal[0], minimal[1], random_reject=False)
-                for retired in retired_indices:
-                    self.walker_group.record(retired[0], retired[1], random_reject=False)
-                retired_indices = []
-                minimal = [{}, float("inf")]
-                indices_lst = self.walker_group.topk(self.re_evalutate_number, modify=True)
-                next_configs = [self.walker_group.to_config(indices) for indices in indices_lst]
-                results = self._cost(configs, indices_lst, use_model)
-                self._log("re-evaluate [%.6f] [ %s]" % (time.time(), "".join("%.6f " % r for r in results)))
-                for indices, result in zip(indices_lst, results):
-                    if result < float("inf"):
-                        self.walker_group.record(indices, result, random_reject=False)
-                self.walker_group.dump_data()        # keep what was measured for the offline trainer
-                self.walker_group.clear_data()
+            if (trial + 1) % remeasure_every == 0:
+                # everything goes back on the heap, and its top points are measured again
+                shelf.pour_into(group)
+                again = group.topk(self.re_evalutate_number, modify=True)
+                costs = self._cost(configs, again, use_model)
+                self._log("re-evaluate [%.6f] [ %s]" % (time.time(), "".join("%.6f " % c for c in costs)))
+                for point, cost in zip(again, costs):
+                    if cost < float("inf"):
+                        group.record(point, cost, random_reject=False)
+                group.dump_data()             # keep what was measured for the offline trainer
+                group.clear_data()
             self._warm_up(1, self.parallel, configs, type_keys, use_model=use_model)
-        self.walker_group.dump_data()
-        self.walker_group.clear_data()
+        group.dump_data()
+        group.clear_data()
         if use_model:
-            if minimal[1] < float("inf"):
-                self.walker_group.record(minimal[0], minimal[1], random_reject=False)
-            for retired in retired_indices:
-                self.walker_group.record(retired[0], retired[1], random_reject=False)
+            shelf.pour_into(group)
             self._finish_with_model(configs, use_model)
-            return self.walker_group.to_config(self.walker_group.top1())
-        if self.walker_group.top1_value() < minimal[1]:
-            best = self.walker_group.top1()
-        else:
-            best = minimal[0]
-        return self.walker_group.to_config(best)
+            return group.to_config(group.top1())
+        return group.to_config(shelf.best_with(group)[0])
 
     def _lowers(self, old_configs, config):
         """True when the templates accept ``config`` in the context of ``old_configs``."""

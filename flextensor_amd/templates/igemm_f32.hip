@@ -9,9 +9,10 @@
 //                             (the transposeB branch, ops.py:1101-1104)
 //           MODE 0 and 2 also run a batch of CG such GEMMs (ops.py:1111-1158)
 //           TA 1 (MODE 0 and 2): A is stored [K][M] (the transposeA branches,
-//           ops.py:1093-1100). Its tile is fetched in vectors along M and
-//           transposed on the way into LDS, where it has the usual [BM][BK]
-//           layout; register-staged pipelines only.
+//           ops.py:1093-1100). On the register-staged pipelines its tile is
+//           fetched in vectors along M and transposed on the way into LDS,
+//           where it has the usual [BM][BK] layout; with DTL it lands as it
+//           lies in memory, [BK][BM], and the fragments are read as scalars.
 //   MODE 1  conv2d NCHW       A = weight [Kout][C*R*S], B = im2col gather of
 //                             the input with zero padding folded into the
 //                             load predicate, N = batch*OH*OW

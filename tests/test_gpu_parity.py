@@ -114,6 +114,28 @@ def test_raw_cabi_launch_and_timing():
         mod.launch((0,), (256,), args)
 
 
+def test_shader_clock_is_read_inside_the_kernels():
+    """The instrumented build of each template (FT_CLKPROBE) computes the same result and reports
+    a plausible sustained clock and workgroup life; the probed plan is a copy, the plan itself is
+    left as it was."""
+    cases = [("gemm", gemm, (256, 256, 256)), ("gemm", gemm_int8, (256, 256, 256)),
+             ("conv2d", depthwise_conv2d, (2, 16, 28, 28, 1, 3, 1, 1, 1)),
+             ("conv2d", conv2d, (2, 16, 14, 14, 32, 3, 1, 1, 1, 1))]
+    for category, func, args in cases:
+        name = {gemm: "gemm", gemm_int8: "gemm_int8", depthwise_conv2d: "depthwise", conv2d: "t"}[func]
+        register(func, category, name, args, "rocm", 0)
+        key = key_of(category, name, args)
+        s, _ = schedule_with_config(key, Config([], None))
+        before = [(k.kernel, dict(k.defines), list(k.args)) for k in s.specs]
+        probe = s.with_clock_probe()
+        assert [(k.kernel, dict(k.defines), list(k.args)) for k in s.specs] == before
+        assert probe.specs[-1].defines["CLKPROBE"] == 1 and probe.specs[-1].args[-1] == ("buf", "clk_probe")
+        assert "clk_probe" in probe.workspaces and "clk_probe" not in s.workspaces
+        clk = Measurer(key, seed=4).shader_clock(s, ms=3.0, warm_ms=30.0)
+        assert clk is not None and 0.5 < clk["ghz"] < 2.6 and clk["ghz_min"] <= clk["ghz"] <= clk["ghz_max"]
+        assert 0.2 < clk["workgroup_us"] < 1000 and clk["workgroups"] >= 1
+
+
 def test_time_limit_abandons_an_overrunning_measurement_and_recovers():
     """The per-candidate time limit (flextensor/measure.py:63-74): a measurement that cannot
     finish inside it comes back as DeviceTimeout (-> inf for the search) without anything being

@@ -571,3 +571,24 @@ def test_schedule_ops_with_config_takes_a_flattened_op_list():
         schedule_ops_with_config(None, list(reversed(op_lst)), Config([], None), "rocm")
     with pytest.raises(RuntimeError):
         schedule_ops_with_config(None, op_lst, Config([], None), "cuda")
+
+
+def test_clock_probe_plan_is_a_copy_with_one_more_argument():
+    """KernelPlan.with_clock_probe: the main kernel gets the FT_CLKPROBE define, a last argument
+    and a [workgroups][2] int64 workspace; every other kernel and the plan itself stay untouched,
+    and the instrumented source compiles for gfx950."""
+    from flextensor_amd.tuned import lookup
+    key = "conv2d_baseline1_(8, 256, 14, 14, 512, 3, 1, 1, 1, 1)_rocm(0)"     # K streaming: workspaces of its own
+    s, _ = schedule_with_config(key, lookup(key))
+    probe = s.with_clock_probe()
+    assert "CLKPROBE" not in s.specs[-1].defines and probe.specs[-1].defines["CLKPROBE"] == 1
+    assert probe.specs[-1].args[:-1] == s.specs[-1].args and probe.specs[-1].args[-1] == ("buf", "clk_probe")
+    nwg = s.specs[-1].grid[0]
+    assert probe.workspaces["clk_probe"] == ((nwg, 2), "int64")
+    assert set(probe.workspaces) == set(s.workspaces) | {"clk_probe"}
+    assert probe.specs[:-1] == s.specs[:-1]
+    assert all(len(code) > 1000 for code in probe.compile())
+    # a plan without a kernel that takes the probe says so
+    from flextensor_amd.plan import KernelPlan
+    with pytest.raises(ValueError):
+        KernelPlan("x", s.bufs, [], {}, None).with_clock_probe()

@@ -1169,6 +1169,54 @@ def test_depthwise_plane_staged_vs_oracle(oracle, args, planes, waves):
                              conv_cfgs(dcfg(1, 8, 9, 20, 1, 4, 1), special=[[0], [0], [2]]))
 
 
+DEGENERATE = [
+    (gemm, "gemm", "gemm", (1, 1, 1)), (gemm, "gemm", "gemm", (1, 17, 3)), (gemm, "gemm", "gemm", (3, 5, 1)),
+    (gemm_int8, "gemm", "gemm_int8", (1, 1, 1)), (gemm_int8, "gemm", "gemm_int8", (2, 3, 5)),
+    (conv2d, "conv2d", "t", (1, 1, 1, 1, 1, 1, 1, 0, 1, 1)),          # one pixel, one channel, one tap
+    (conv2d, "conv2d", "t", (1, 3, 5, 5, 2, 3, 1, 0, 1, 1)),          # 3x3 output
+    (conv2d, "conv2d", "t", (1, 2, 3, 3, 4, 3, 1, 1, 1, 2)),          # one channel per group: the depthwise kernel
+    (depthwise_conv2d, "conv2d", "depthwise", (1, 1, 1, 1, 1, 1, 1, 0, 1)),
+    (depthwise_conv2d, "conv2d", "depthwise", (1, 3, 3, 3, 2, 3, 1, 1, 1)),
+    (depthwise_conv2d, "conv2d", "depthwise", (2, 2, 5, 7, 1, 3, 2, 0, 1)),
+]
+
+
+@pytest.mark.parametrize("func,category,name,args", DEGENERATE)
+def test_smallest_extents(oracle, func, category, name, args):
+    """Extents of one and a few: every tile is an edge tile, most lanes idle, K far below one MFMA step."""
+    register(func, category, name, args, "rocm", 0)
+    key = key_of(category, name, args)
+    ops, bufs = TASK_TABLE[key].func(*args)
+    host = seeded_inputs(bufs, seed=sum(args) + 1)
+    out = run_plan(key, Config([], None), host)
+    if func is gemm_int8:
+        assert np.array_equal(out, oracle.gemm_i8_c(host[0], host[1]))
+        ref = oracle.gemm_i8_np(host[0], host[1])
+    elif func is gemm:
+        ref = oracle.gemm_f32_c(host[0], host[1])
+    elif func is conv2d:
+        ref = oracle.conv2d_nchw_c(host[0], host[1], args[6], args[7], args[8], args[9])
+    else:
+        ref = oracle.depthwise_nchw_c(host[0], host[1], args[6], args[7], args[8])
+    assert out.shape == np.asarray(ref).shape
+    assert rel(out, ref) <= TOL
+    # the default-schedule kernels the search gates candidates against
+    tdt = {"float32": torch.float32, "int32": torch.int32}[bufs[-1].dtype]
+    dev = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in host]
+    gate = torch.full(bufs[-1].shape, -77, dtype=tdt, device="cuda")
+    run_default_schedule(ops, dev + [gate], stream=current_stream())
+    torch.cuda.synchronize()
+    assert rel(gate.cpu().numpy(), ref) <= TOL
+
+
+def test_empty_extents_are_refused_on_the_host():
+    for func, category, name, args in ((gemm, "gemm", "gemm", (0, 4, 4)), (gemm, "gemm", "gemm", (4, 0, 4)),
+                                       (gemm_int8, "gemm", "gemm_int8", (4, 4, 0))):
+        with pytest.raises(Exception):
+            register(func, category, name, args, "rocm", 0)
+            schedule_with_config(key_of(category, name, args), Config([], None))
+
+
 def test_default_schedule_kernels_vs_oracle(oracle):
     """The plain kernels every candidate is gated against are themselves right."""
     s = current_stream()

@@ -15,6 +15,14 @@ sink a shift into the arm of a select; the depthwise kernels therefore compute
 their shifts before any select, and this check looks for a DPP instruction
 between an ``s_and_saveexec`` and the instruction that restores ``exec``.
 
+4. Register copies ahead of an execution-mask restore. The join block of a divergent
+``if`` begins with ``s_or_b64 exec, exec, <saved>``. Under register pressure the compiler
+has placed its own copies of unrelated live values (live-range splits, spills into
+accumulation registers) at the top of that block, in front of the restore, where only the
+lanes that took the branch execute them: the other lanes keep stale registers. The sign in
+the assembly text is a basic block whose vector instructions up to the restore are nothing
+but register-to-register copies.
+
 For 1: the hardware does not interlock this case; the compiler pads it with s_nop,
 but its padding follows the control-flow graph with a visited set per block
 and can lose a short path. This module rebuilds the graph from the assembly
@@ -226,6 +234,41 @@ def find_masked_lane_shifts(asm_text, kernel):
     return found, insts
 
 
+BLOCK_START = re.compile(r"^\s*(\.LBB\d+_\d+:|; %bb\.\d+:)")
+VECTOR = re.compile(r"^(v_|ds_|buffer_|global_|scratch_|flat_)")
+LANE_ACCESS = ("v_readlane", "v_writelane")          # SGPR spills: these ignore exec
+COPY = re.compile(r"^(v_mov_b32_e32 v\d+, v\d+|v_mov_b64_e32 v\[\d+:\d+\], v\[\d+:\d+\]"
+                  r"|v_accvgpr_(write|read|mov)_b32 [av]\d+, [av]\d+)$")
+
+
+def find_copies_ahead_of_exec_restore(asm_text, kernel):
+    """[(line number of the restore, [copy instructions])] for basic blocks in which
+    nothing but register copies stands between the block's start and its
+    ``s_or_b64 exec, exec, ...``. (A block that does real work under the narrowed mask
+    and then restores it, a predicated store merged with its join block, is the
+    ordinary case and is not reported.)"""
+    lines = asm_text.split("\n")
+    start = next(i for i, l in enumerate(lines) if l.startswith(kernel + ":"))
+    found, vec = [], []
+    for n, l in enumerate(lines[start + 1:], start + 2):
+        if l.startswith(".Lfunc_end"):
+            break
+        if BLOCK_START.match(l):
+            vec = []
+            continue
+        s = l.split(";")[0].strip()
+        if not s or s.startswith(".") or s.endswith(":"):
+            continue
+        name = s.split(None, 1)[0]
+        if name == "s_or_b64" and re.match(r"\s*exec\b", s[len(name):]):
+            if vec and all(COPY.match(x) for x in vec):
+                found.append((n, list(vec)))
+            vec = []
+        elif VECTOR.match(name) and not name.startswith(LANE_ACCESS):
+            vec.append(s)
+    return found
+
+
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
@@ -248,17 +291,21 @@ def assembly_of(spec, workdir=None):
 def check_plan(plan):
     """[(kernel, first instruction, second instruction, detail)] over the kernels of a plan:
     early reads of MFMA results (detail = issue slots between), arrival counts of the
-    K-streaming exchange that do not wait for the slot stores (detail = "arrival"), and in
-    the depthwise kernels DPP lane shifts under a narrowed exec mask (detail = "masked shift")."""
+    K-streaming exchange that do not wait for the slot stores (detail = "arrival"), in
+    the depthwise kernels DPP lane shifts under a narrowed exec mask (detail = "masked shift"),
+    and in all of them register copies ahead of an exec restore (detail = "masked copy";
+    the two instructions are then the first copy and the line number of the restore)."""
     out = []
     for spec in plan.specs:
-        if spec.kernel == "depthwise_f32":
-            found, insts = find_masked_lane_shifts(assembly_of(spec), spec.kernel)
-            out.extend((spec.kernel, insts[i], insts[j], "masked shift") for i, j in found)
-            continue
-        if spec.kernel not in ("igemm_f32", "gemm_i8"):
+        if spec.kernel not in ("igemm_f32", "gemm_i8", "depthwise_f32"):
             continue
         text = assembly_of(spec)
+        out.extend((spec.kernel, (copies[0], ""), ("s_or_b64", "exec, line %d" % n), "masked copy")
+                   for n, copies in find_copies_ahead_of_exec_restore(text, spec.kernel))
+        if spec.kernel == "depthwise_f32":
+            found, insts = find_masked_lane_shifts(text, spec.kernel)
+            out.extend((spec.kernel, insts[i], insts[j], "masked shift") for i, j in found)
+            continue
         found, insts = find_early_reads(text, spec.kernel)
         out.extend((spec.kernel, insts[i], insts[j], used) for i, j, used in found)
         if spec.defines.get("SK_PER", 0):
@@ -287,6 +334,8 @@ def main(argv):
             bad += 1
             if used == "arrival":
                 print("UNORDERED ARRIVAL %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
+            elif used == "masked copy":
+                print("REGISTER COPY AHEAD OF AN EXEC RESTORE %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
             elif used == "masked shift":
                 print("LANE SHIFT UNDER A NARROWED EXEC MASK %s %s: %s %s -> %s %s" % ((key, kernel) + mfma + reader))
             else:

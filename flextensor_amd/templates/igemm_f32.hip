@@ -700,11 +700,13 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
     const i32x4 desc_a = descriptor(A, (unsigned)A_BYTES);
     const i32x4 desc_b = descriptor(B, (unsigned)B_BYTES);
     /* The descriptor, the LDS address and the scalar offset are wave-uniform by construction.
-     * With more than two buffers inside the K-streaming segment loop (a buffer index carried around
-     * a loop that has lane-dependent exits) the compiler no longer sees that and would hand the
-     * instruction vector registers, so there it is told; everywhere else it knows, and telling it
-     * anyway costs instructions in the main loop. */
-#if SK_PER > 0 && STAGES > 2
+     * With more than two buffers the buffer index is carried around the tile loop as a variable,
+     * and in some shapes of that loop (inside the K-streaming segment loop with its lane-dependent
+     * exits; in a workgroup of one wavefront) the compiler keeps it in a vector register and would
+     * hand the instruction vector operands, so there it is told. With one or two buffers the index
+     * is a constant or a bit of the tile counter, the compiler knows, and telling it anyway costs
+     * instructions in the main loop. */
+#if STAGES > 2
 #define DMA_UNIFORM(x) __builtin_amdgcn_readfirstlane((int)(x))
     auto uniform4 = [](const i32x4& v) {
         i32x4 r;
@@ -774,9 +776,10 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int rs = k % (CR * CS);
             const int ih = px_h[e] + (rs / CS) * CDILH;
             const int iw = px_w[e] + (rs % CS) * CDILW;
-            bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-            if (KP != K) ok = ok && (k < K);
-            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
+            bool ok = px_ok[e] & ((unsigned)ih < (unsigned)CH) & ((unsigned)iw < (unsigned)CW);
+            if (KP != K) ok = ok & (k < K);
+            const unsigned off = (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u;
+            const unsigned vo = ok ? off : OOB;      /* a select of two values, no branch (see a_voff) */
             dma4(desc_b, dst, vo, 0);
 #endif
 #endif
@@ -792,19 +795,27 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         dma_tile_b(kt, buf, part, nparts);
     };
 #endif
+    /* Every offset below is computed for all lanes and then chosen against the out-of-range
+     * constant: a select of two values, never "compute it if in range". The second form becomes a
+     * divergent branch around the arithmetic, and under register pressure the compiler has put its
+     * own register-to-register copies of unrelated live values (live-range splits) into the join
+     * block ahead of the instruction that restores the execution mask, so lanes that were out of
+     * range kept stale registers and later tiles were gathered from wrong rows. */
 #pragma unroll
     for (int e = 0; e < EA; ++e) {
 #if TA
         /* a_row = k inside the tile, a_col = first of AV consecutive rows m (M % AV == 0) */
         const int m = m0 + a_col[e];
         bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
-        if (M % BM != 0) ok = ok && (m < M);
-        a_voff[e] = ok ? (unsigned)((gi * K + a_row[e]) * M + m) * 4u : OOB;
+        if (M % BM != 0) ok = ok & (m < M);
+        const unsigned off = (unsigned)((gi * K + a_row[e]) * M + m) * 4u;
+        a_voff[e] = ok ? off : OOB;
 #else
         const int m = m0 + a_row[e];
         bool ok = (A_CHUNKS % NT == 0) || (tid + e * NT < A_CHUNKS);
-        if (M % BM != 0) ok = ok && (m < M);
-        a_voff[e] = ok ? (unsigned)((gi * M + m) * K + a_col[e]) * 4u : OOB;
+        if (M % BM != 0) ok = ok & (m < M);
+        const unsigned off = (unsigned)((gi * M + m) * K + a_col[e]) * 4u;
+        a_voff[e] = ok ? off : OOB;
 #endif
     }
 #if DTL
@@ -817,7 +828,7 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
 #pragma unroll
     for (int e = 0; e < EB; ++e) {
         const int n = n0 + b_col[e];
-        px_ok[e] = (n < N) && (tid + e * NT < B_CHUNKS);
+        px_ok[e] = (n < N) & (tid + e * NT < B_CHUNKS);
         const int nn = px_ok[e] ? n : 0;
         const int b = nn / OHW;
         const int p = nn % OHW;
@@ -831,12 +842,14 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         bool ok = (B_CHUNKS % NT == 0) || (tid + e * NT < B_CHUNKS);
 #if MODE == 2
         const int n = n0 + b_row[e];
-        if (N % BN != 0) ok = ok && (n < N);
-        b_voff[e] = ok ? (unsigned)((gi * N + n) * K + b_col[e]) * 4u : OOB;
+        if (N % BN != 0) ok = ok & (n < N);
+        const unsigned off = (unsigned)((gi * N + n) * K + b_col[e]) * 4u;
+        b_voff[e] = ok ? off : OOB;
 #elif MODE == 0
         const int n = n0 + b_col[e];
-        if (N % BN != 0) ok = ok && (n < N);
-        b_voff[e] = ok ? (unsigned)((gi * K + b_row[e]) * N + n) * 4u : OOB;
+        if (N % BN != 0) ok = ok & (n < N);
+        const unsigned off = (unsigned)((gi * K + b_row[e]) * N + n) * 4u;
+        b_voff[e] = ok ? off : OOB;
 #elif KHOIST
 #if BROW_LINEAR
         /* every element of this lane is the same pixel, BROW_STEP rows of the tile further down:
@@ -847,15 +860,17 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
         const int cl = cl0 + (e * BROW_STEP) / (CR * CS) + (rsx >= CR * CS ? 1 : 0);
         const int ih = px_h[0] + (rs / CS) * CDILH;
         const int iw = px_w[0] + (rs % CS) * CDILW;
-        ok = ok && px_ok[0] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-        b_voff[e] = ok ? (unsigned)(px_off[0] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
+        ok = ok & px_ok[0] & ((unsigned)ih < (unsigned)CH) & ((unsigned)iw < (unsigned)CW);
+        const unsigned off = (unsigned)(px_off[0] + cl * (CH * CW) + ih * CW + iw) * 4u;
+        b_voff[e] = ok ? off : OOB;
 #else
         const int cl = b_row[e] / (CR * CS);
         const int rs = b_row[e] % (CR * CS);
         const int ih = px_h[e] + (rs / CS) * CDILH;
         const int iw = px_w[e] + (rs % CS) * CDILW;
-        ok = ok && px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-        b_voff[e] = ok ? (unsigned)(px_off[e] + cl * (CH * CW) + ih * CW + iw) * 4u : OOB;
+        ok = ok & px_ok[e] & ((unsigned)ih < (unsigned)CH) & ((unsigned)iw < (unsigned)CW);
+        const unsigned off = (unsigned)(px_off[e] + cl * (CH * CW) + ih * CW + iw) * 4u;
+        b_voff[e] = ok ? off : OOB;
 #endif
 #else
         b_voff[e] = OOB;  /* recomputed for every tile */
@@ -901,9 +916,10 @@ void igemm_f32(const float* __restrict__ A, const float* __restrict__ B,
             const int rs = k % (CR * CS);
             const int ih = px_h[e] + (rs / CS) * CDILH;
             const int iw = px_w[e] + (rs % CS) * CDILW;
-            bool ok = px_ok[e] && (unsigned)ih < (unsigned)CH && (unsigned)iw < (unsigned)CW;
-            if (KP != K) ok = ok && (k < K);
-            const unsigned vo = ok ? (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u : OOB;
+            bool ok = px_ok[e] & ((unsigned)ih < (unsigned)CH) & ((unsigned)iw < (unsigned)CW);
+            if (KP != K) ok = ok & (k < K);
+            const unsigned off = (unsigned)(px_off[e] + c * (CH * CW) + ih * CW + iw) * 4u;
+            const unsigned vo = ok ? off : OOB;      /* a select of two values, no branch (see a_voff) */
             breg[set][e] = LOAD_B(rsrc_b, vo, 0);
 #endif
         }

@@ -435,6 +435,11 @@ def test_gemm_transpose_b_direct_to_lds(oracle):
     ((8, 64, 7, 7, 96, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=32, bk=16, st=6), [-1, 8]),
     ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=1, rn=1, mf=32, bk=72, st=6), [0, 0]),
     ((8, 512, 7, 7, 2048, 1, 1, 0, 1, 1), dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=32, st=7, ks=1), [-1, 0]),
+    # the same in workgroups of one wavefront (the ring's buffer index once reached the
+    # load instruction in a vector register there, and the kernel did not assemble)
+    ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=1, rm=2, wn=1, rn=5, mf=16, bk=16, st=7), [-1, 0]),
+    ((2, 32, 14, 14, 64, 3, 1, 1, 1, 4), dict(wm=1, rm=1, wn=1, rn=3, mf=32, bk=16, st=6), [-1, 0]),
+    ((2, 32, 16, 16, 64, 3, 1, 0, 1, 4), dict(wm=1, rm=1, wn=1, rn=4, mf=16, bk=16, st=6), [-1, 0]),
     # unpadded B rows permuted against bank conflicts: every row width / MFMA shape of the permutation
     ((2, 16, 14, 14, 32, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=2, rn=1, mf=16, bk=16, st=5), [-1, 0]),    # 32 floats, 16x16x4
     ((2, 16, 14, 14, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=1, wn=4, rn=1, mf=16, bk=16, st=5), [-1, 0]),    # 64 floats, 16x16x4
@@ -869,6 +874,10 @@ CONV_CASES = [
     # end one tile and begin the next (an early version of the exchange summed this one wrong)
     ((1, 64, 56, 56, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=2, wn=2, rn=1, mf=16, bk=16, st=3, ks=1)),
     ((1, 64, 56, 56, 64, 3, 1, 1, 1, 1), dict(wm=2, rm=2, wn=2, rn=1, mf=16, bk=16, st=2, ks=2)),
+    # one wavefront, 224 columns, two register sets of 56 gathered elements, 112 accumulators: every
+    # register in use (the compiler once split live ranges inside the divergent address arithmetic
+    # of this kernel and lanes outside the image kept stale rows)
+    ((3, 6, 11, 11, 20, 3, 1, 2, 2, 1), dict(wm=1, rm=1, wn=1, rn=7, mf=32, bk=16, st=3)),
 ]
 
 

@@ -189,6 +189,61 @@ def test_lane_shift_checker_flags_a_shift_behind_a_narrowed_mask():
     assert found == []
 
 
+JOIN = """k:
+\tv_bfrev_b32_e32 v60, 1
+\ts_and_saveexec_b64 s[18:19], s[34:35]
+; %%bb.229:
+\tv_mul_i32_i24_e32 v56, 11, v56
+\tv_lshl_add_u32 v60, v56, 2, v59
+; %%bb.230:
+%s\ts_or_b64 exec, exec, s[18:19]
+\tbuffer_load_dword a233, v60, s[56:59], 0 offen
+\ts_and_saveexec_b64 s[4:5], s[6:7]
+\ts_cbranch_execz .LBB0_2
+; %%bb.231:
+\tv_mov_b32_e32 v5, v7
+\tglobal_store_dword v[126:127], v5, off
+.LBB0_2:
+\ts_or_b64 exec, exec, s[4:5]
+\ts_endpgm
+.Lfunc_end0:
+"""
+
+
+def test_copy_checker_flags_copies_between_a_join_block_and_its_exec_restore():
+    """The form the compiler produced in a register-starved gather kernel: copies of unrelated live
+    values at the top of the join block, ahead of the restore, so that only the lanes of the branch
+    execute them. A block that works under the mask and restores it at its own end is not that."""
+    split = "\tv_accvgpr_write_b32 a18, v240\n\tv_mov_b32_e32 v28, v93\n\ts_mov_b64 s[42:43], s[40:41]\n"
+    found = isa_hazards.find_copies_ahead_of_exec_restore(JOIN % split, "k")
+    assert [copies for _, copies in found] == [["v_accvgpr_write_b32 a18, v240", "v_mov_b32_e32 v28, v93"]]
+    assert isa_hazards.find_copies_ahead_of_exec_restore(JOIN % "", "k") == []
+    # SGPR spills into lanes ignore exec and do not count
+    lanes = "\tv_writelane_b32 v254, s18, 46\n"
+    assert isa_hazards.find_copies_ahead_of_exec_restore(JOIN % lanes, "k") == []
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_register_starved_gather_kernel_has_no_divergent_address_arithmetic():
+    """224 columns, two register sets of 56 gathered elements each, 112 accumulators: the kernel in
+    which the copies were found (wrong rows in the tiles loaded inside the loop). The offsets are
+    selects now, so the address set-up has no divergent branch for the compiler to split around."""
+    from flextensor_amd.task import Task, conv2d, register
+    args = (3, 6, 11, 11, 20, 3, 1, 2, 2, 1)
+    register(conv2d, "conv2d", "rnd", args, "rocm", 0)
+    key = Task("conv2d", "rnd", None, args, "rocm", 0).key
+    c = {k: [] for k in KEYS}
+    c.update(fuse=[[8]], spatial=[[1, 1, 1, 32], [2, 1, 7, 32]], reduce=[[1, 4, 16]], reorder=[[0, 1, 0]],
+             unroll=[[3, 1]])
+    g = {k: [] for k in KEYS}
+    g["inline"], g["special"] = [[1, 0]], [[4, -1]]
+    plan, _ = schedule_with_config(key, Config([{k: [] for k in KEYS}, c], g))
+    text = isa_hazards.assembly_of(plan.specs[-1])
+    first_mfma = text.index("v_mfma")
+    assert "s_and_saveexec" not in text[:first_mfma]
+    assert isa_hazards.check_plan(plan) == []
+
+
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 @pytest.mark.parametrize("special", [[[1], [0], [0], [1], [2]],      # row exchange (the shipped variant)
                                      [[1], [0], [0], [1], [3]],      # ragged last span
@@ -212,7 +267,8 @@ def test_depthwise_lane_shifts_run_with_every_lane_switched_on(special):
 def test_random_points_of_the_spaces_pass_the_static_checks(shape_index):
     """The generated assembly of points drawn at random from the schedule spaces (the same points
     the device parity test runs): no accumulator read before the matrix core has written it, no
-    arrival counted ahead of the slot stores, no lane shift under a narrowed exec mask."""
+    arrival counted ahead of the slot stores, no lane shift under a narrowed exec mask, no register
+    copies between a join block's start and its exec restore."""
     from random_points import point
     for number in (0, 4):
         kind, key, args, configs, plan = point(shape_index, number)

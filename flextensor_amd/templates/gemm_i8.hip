@@ -44,6 +44,13 @@
 //               next group's MFMAs cover the distance to the read: the stores of C
 //               start a tile's time before the workgroup's last MFMA instead of
 //               behind it
+//   SPLITK      grid-level split of K: SPLITK workgroups per tile, each over a
+//               contiguous range of K; the partial sums meet in C (zero-filled by a
+//               kernel in front) through integer atomic adds, which are exact and
+//               order-independent, so the result stays bit-exact and repeatable
+//   WAVES_K     split of K inside the workgroup: WAVES_K groups of WAVES_M x WAVES_N
+//               wavefronts, each with its own LDS tiles and its own range of K; the
+//               groups' accumulators are summed through LDS and group 0 stores
 //   CVEC        1: the MFMA operands are swapped (the core computes the
 //               transposed tile), so a lane holds four consecutive columns of
 //               one row of C and writes them with one 128-bit store
@@ -88,6 +95,16 @@
 #else
 #define EARLYST 0
 #endif
+#ifdef FT_SPLITK
+#define SPLITK FT_SPLITK
+#else
+#define SPLITK 1
+#endif
+#ifdef FT_WAVES_K
+#define WAVES_K FT_WAVES_K
+#else
+#define WAVES_K 1
+#endif
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
@@ -113,7 +130,8 @@ typedef i32x4 acc_t;
 
 #define BM (WAVES_M * REP_M * MFMA)
 #define BN (WAVES_N * REP_N * MFMA)
-#define NT (WAVES_M * WAVES_N * 64)
+#define NT (WAVES_M * WAVES_N * 64)      /* threads of one k-group */
+#define NTW (NT * WAVES_K)               /* threads of the workgroup */
 #define CRW (BK / 16)             /* 16-byte chunks per LDS row */
 #if PAD < 0
 #define SROW (BK)                 /* LDS row stride in bytes */
@@ -137,7 +155,10 @@ typedef i32x4 acc_t;
  * partly beyond it (those bytes are the next row's, not zeros): the chunk is
  * then put together from dword loads (K % 4 == 0) or byte loads, each with its
  * own predicate. Register-staged pipelines only. */
-#define KT (KP / BK)
+#define KT (KP / BK / (SPLITK * WAVES_K))      /* tiles of one k-group (host checks divisibility) */
+#if EARLYST && (SPLITK > 1 || WAVES_K > 1)
+#error "early stores write finished sums: no K division"
+#endif
 
 #if BK % MFMA_K != 0
 #error "BK must be a multiple of the MFMA K extent"
@@ -177,15 +198,31 @@ typedef __attribute__((address_space(3))) void lds_void;
 #define CLK_END do { } while (0)
 #endif
 
-extern "C" __global__ __launch_bounds__(NT)
+#define A_TILE_BYTES (BM * SROW)
+#define B_TILE_BYTES (BN * SROW)
+#define TILE_BYTES (WAVES_K * STAGES * (A_TILE_BYTES + B_TILE_BYTES))
+#define RED_BYTES ((WAVES_K - 1) * NT * REP_M * REP_N * NACC * 4)
+#define SMEM_BYTES (TILE_BYTES > RED_BYTES ? TILE_BYTES : RED_BYTES)
+
+extern "C" __global__ __launch_bounds__(NTW)
 void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ B,
              int* __restrict__ C CLK_PARAM)
 {
     CLK_BEGIN
+#if WAVES_K > 1
+    /* every k-group has its own tiles; the memory is reused for the sum of the groups */
+    __shared__ __attribute__((aligned(16))) signed char smem[SMEM_BYTES];
+    const int kg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / NT));
+    const int tid = threadIdx.x - kg * NT;          /* thread index inside the k-group */
+    signed char (*As)[A_TILE_BYTES] = reinterpret_cast<signed char (*)[A_TILE_BYTES]>(smem + kg * STAGES * A_TILE_BYTES);
+    signed char (*Bs)[B_TILE_BYTES] = reinterpret_cast<signed char (*)[B_TILE_BYTES]>(
+        smem + WAVES_K * STAGES * A_TILE_BYTES + kg * STAGES * B_TILE_BYTES);
+#else
     __shared__ __attribute__((aligned(16))) signed char As[STAGES][BM * SROW];
     __shared__ __attribute__((aligned(16))) signed char Bs[STAGES][BN * SROW];
-
+    const int kg = 0;
     const int tid = threadIdx.x;
+#endif
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave / WAVES_N;
@@ -193,11 +230,18 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     const int li = lane % MFMA;
     const int lg = lane / MFMA;
 
-    const int nblk = TILES_M * TILES_N;
+    const int nblk = TILES_M * TILES_N * SPLITK;
     int bid = blockIdx.x;
 #if XCD_REMAP
     if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
 #endif
+#if SPLITK > 1
+    const int kz = bid / (TILES_M * TILES_N);       /* which part of K */
+    bid = bid % (TILES_M * TILES_N);
+#else
+    const int kz = 0;
+#endif
+    const int kbase = (kz * WAVES_K + kg) * (KT * BK);     /* first k of this group's range */
     const int grp = bid / (GROUP_M * TILES_N);
     const int first_m = grp * GROUP_M;
     const int gsz = (TILES_M - first_m) < GROUP_M ? (TILES_M - first_m) : GROUP_M;
@@ -280,7 +324,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     };
 
     auto load_global = [&](int kt, int set) {
-        const int k0 = kt * BK;
+        const int k0 = kbase + kt * BK;
 #pragma unroll
         for (int e = 0; e < EA; ++e) {
             unsigned vo = a_voff[e];
@@ -333,11 +377,16 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
                 i32x4 v4;
                 v4[0] = acc[i][j][4 * q + 0]; v4[1] = acc[i][j][4 * q + 1];
                 v4[2] = acc[i][j][4 * q + 2]; v4[3] = acc[i][j][4 * q + 3];
+#if SPLITK > 1
+#pragma unroll
+                for (int x = 0; x < 4; ++x) atomicAdd(C + (size_t)m * N + n + x, v4[x]);
+#else
                 i32x4* dst = reinterpret_cast<i32x4*>(C + (size_t)m * N + n);
 #if NT_STORE
                 __builtin_nontemporal_store(v4, dst);
 #else
                 *dst = v4;
+#endif
 #endif
             }
         }
@@ -355,7 +404,9 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
             if (M % BM != 0) ok = ok && (m < M);
             if (N % BN != 0) ok = ok && (n < N);
             if (ok) {
-#if NT_STORE
+#if SPLITK > 1
+                atomicAdd(C + (size_t)m * N + n, acc[i][j][v]);
+#elif NT_STORE
                 __builtin_nontemporal_store(acc[i][j][v], C + (size_t)m * N + n);
 #else
                 C[(size_t)m * N + n] = acc[i][j][v];
@@ -412,7 +463,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
                          :: "s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so) : "memory", "m0");
         };
         auto dma_tile = [&](int kt, int buf) {
-            const int k0 = kt * BK;
+            const int k0 = kbase + kt * BK;
 #pragma unroll
             for (int e = 0; e < EA; ++e) {
                 unsigned vo = a_voff[e];
@@ -456,7 +507,7 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
                 fB[set][g - REP_M] = *reinterpret_cast<const i32x4*>(&Bs[buf][(brow + (g - REP_M) * MFMA) * SROW + PCOL(brow + (g - REP_M) * MFMA, kk + 16 * lg)]);
         };
         auto dma_one = [&](int kt, int buf, int e) {
-            const int k0 = kt * BK;
+            const int k0 = kbase + kt * BK;
             if (e < EA) {
                 unsigned vo = a_voff[e];
                 if (KP != K) vo = (k0 + a_col[e] < K) ? vo : OOB;
@@ -688,6 +739,33 @@ void gemm_i8(const signed char* __restrict__ A, const signed char* __restrict__ 
     asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
+#if WAVES_K > 1
+    /* ---- sum the k-groups' partial tiles through LDS ---- */
+    __syncthreads();             /* every group has read its last fragments: tile memory is free */
+    if (kg > 0) {
+        int* red = reinterpret_cast<int*>(smem) + (kg - 1) * (NT * REP_M * REP_N * NACC);
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v)
+                    red[((i * REP_N + j) * NACC + v) * NT + tid] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (kg > 0) return;
+#pragma unroll
+    for (int g = 1; g < WAVES_K; ++g) {
+        const int* red = reinterpret_cast<const int*>(smem) + (g - 1) * (NT * REP_M * REP_N * NACC);
+#pragma unroll
+        for (int i = 0; i < REP_M; ++i)
+#pragma unroll
+            for (int j = 0; j < REP_N; ++j)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v)
+                    acc[i][j][v] += red[((i * REP_N + j) * NACC + v) * NT + tid];
+    }
+#endif
 #if !EARLYST
 #pragma unroll
     for (int i = 0; i < REP_M; ++i)

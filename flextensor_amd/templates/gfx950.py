@@ -195,7 +195,7 @@ def _gemm_space(view):
     space.add_subspace("split_m_0", TileSplitSpace(view.M, reps=reps), "spatial")
     space.add_subspace("split_n_1", TileSplitSpace(view.N, reps=reps), "spatial")
     bks = I8_BK if i8 else F32_BK
-    max_split = 1 if i8 else 16
+    max_split = 16
 
     def keep(e):
         return e[2] in bks and e[0] <= max_split
@@ -214,7 +214,8 @@ def _gemm_space(view):
                        "unroll")
     space.add_subspace("group_m", EnumSpace([[1], [2], [4], [8], [16]]), "fuse")
     # [xcd remap, K partitions inside the workgroup (1) or across workgroups (0)]
-    space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0]] if i8 else
+    # the third number: balanced K streaming with that many workgroups per compute unit (fp32 only)
+    space.add_subspace("xcd_remap", EnumSpace([[1, 0, 0], [0, 0, 0], [1, 1, 0], [0, 1, 0]] if i8 else
                                             [[1, 0, 0], [0, 0, 0], [1, 1, 0], [0, 1, 0], [1, 0, 1], [1, 0, 2]]),
                        "reorder")
     return space
@@ -355,8 +356,6 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
     i8 = view.dtype == "int8"
     waves_k = 1
     if in_wg and splitk > 1:
-        if i8:
-            raise InvalidConfig("int8 GEMM does not split K")
         waves_k, splitk = splitk, 1
 
     if mfm != mfn or mfm not in (16, 32):
@@ -380,8 +379,10 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
              REP_N=rn, BK=bk, STAGES=stages, GROUP_M=group_m, XCD_REMAP=xcd)
 
     if i8:
-        if splitk != 1 or stream_k:
-            raise InvalidConfig("int8 GEMM does not split K across workgroups")
+        if stream_k:
+            # the grid-level split (integer atomics: exact, any order) and the in-workgroup split
+            # cover the int8 operator; the balanced K streaming protocol is an fp32 path
+            raise InvalidConfig("int8 GEMM splits K across workgroups or wavefront groups, not by K streaming")
         mfma_k = 32 if mfm == 32 else 64
         if bk % mfma_k != 0:
             raise InvalidConfig("BK must be a multiple of the MFMA K extent")
@@ -405,7 +406,7 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
                                         "and enough MFMAs per k-step to interleave with")
         elif (ceil_div(bm * bk // 16, nt) + ceil_div(bn * bk // 16, nt)) * 4 * pd > 160:
             raise InvalidConfig("global->LDS staging needs too many registers")
-        lds = stages * (bm + bn) * (bk + max(pad, 0))
+        lds = max(waves_k * stages * (bm + bn) * (bk + max(pad, 0)), (waves_k - 1) * nt * nacc * 4)
         if lds > LDS_BYTES:
             raise InvalidConfig("LDS tile needs %d bytes" % lds)
         # nt_store: bit 0 = non-temporal stores, bit 1 = transposed MFMA so that lanes store 128-bit rows,
@@ -413,8 +414,9 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
         store_mode = int(_special(special, "nt_store")[0])
         if store_mode & 2 and view.N % 4 != 0:
             raise InvalidConfig("128-bit C stores need N to be a multiple of 4")
-        if store_mode & 4 and (depth != 7 or bk != 2 * mfma_k or kp // bk < 2):
-            raise InvalidConfig("early stores come with pipeline depth 7, two k-steps per tile, two tiles or more")
+        if store_mode & 4 and (depth != 7 or bk != 2 * mfma_k or kp // bk < 2 or splitk * waves_k != 1):
+            raise InvalidConfig("early stores come with pipeline depth 7, two k-steps per tile, two tiles or more, "
+                                "and an undivided K")
         D.update(PAD=pad, PD=pd, FRAGPF=1 if depth == 5 else 0, NT_STORE=store_mode & 1)
         if depth >= 6:
             D.update(DTL=depth - 5)
@@ -422,10 +424,20 @@ def _lower_gemm(op, config, special, out_name, in_names, materialized_pad=False,
             D.update(CVEC=1)
         if store_mode & 4:
             D.update(EARLYST=1)
-        grid = (gm * gn, 1, 1)
-        spec = KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt, 1, 1),
-                          [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)])
-        return [spec]
+        specs = []
+        if splitk > 1:
+            # partial sums meet in C: zero it first (the fill writes zero bit patterns, whatever the type)
+            D.update(SPLITK=splitk)
+            nout = view.M * view.N
+            specs.append(KernelSpec("elementwise.hip", "fill_zero_f32", {},
+                                    (min(ceil_div(ceil_div(nout, 4), 256), 2048), 1, 1), (256, 1, 1),
+                                    [("buf", out_name), ("i32", nout)], note="split-K zero fill"))
+        if waves_k > 1:
+            D.update(WAVES_K=waves_k)
+        grid = (gm * gn * splitk, 1, 1)
+        specs.append(KernelSpec("gemm_i8.hip", "gemm_i8", D, grid, (nt * waves_k, 1, 1),
+                                [("buf", in_names[0]), ("buf", in_names[1]), ("buf", out_name)]))
+        return specs
 
     kblk = 4 * (64 // mfm)
     if bk % kblk != 0:
@@ -859,7 +871,7 @@ def seed_configs(op, limit=24):
                     cfg["fuse"] = [[8]]
                     cfg["reorder"] = [[1, 0, stream]]
                     out.append(cfg)
-                if not i8 and depth == depths[0] and stream == 0 and tiles * 2 <= NUM_CUS:
+                if depth == depths[0] and stream == 0 and tiles * 2 <= NUM_CUS:
                     # few tiles and a long K (weights streamed past a small image): K parts across
                     # workgroups, as many as fill the compute units
                     split = 1

@@ -834,6 +834,51 @@ def test_gemm_int8_k_not_a_multiple_of_16(oracle, M, K, N, kn):
         schedule_with_config(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **dict(kn, st=6))], None))
 
 
+@pytest.mark.parametrize("M,K,N,kn", [
+    # K across workgroups: integer atomic adds into a zero-filled C
+    (136, 512, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64, sk=4)),                # ragged, register-staged
+    (64, 1024, 96, dict(wm=1, rm=2, wn=1, rn=2, mf=16, bk=128, sk=8, st=5)),         # fragment prefetch, one tile per part
+    (200, 1000, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, sk=4, st=3)),        # K tail in the last part only
+    (256, 2048, 256, dict(wm=2, rm=2, wn=2, rn=2, mf=32, bk=128, sk=4, st=7)),       # tiles straight into LDS
+    (256, 2048, 256, dict(wm=2, rm=4, wn=2, rn=4, mf=16, bk=128, sk=2, st=8)),       # written-out instruction order
+    (80, 333, 96, dict(wm=1, rm=1, wn=2, rn=1, mf=32, bk=128, sk=3, st=2)),          # odd K: byte loads in every part
+    # K across wavefront groups of one workgroup: summed through LDS
+    (136, 512, 72, dict(wm=2, rm=1, wn=1, rn=1, mf=32, bk=64, sk=4, wk=1)),
+    (64, 1024, 96, dict(wm=1, rm=2, wn=1, rn=2, mf=16, bk=128, sk=8, wk=1, st=5)),
+    (200, 1000, 136, dict(wm=2, rm=2, wn=1, rn=2, mf=16, bk=64, sk=4, wk=1, st=3)),
+    (128, 2048, 128, dict(wm=2, rm=2, wn=2, rn=2, mf=16, bk=128, sk=4, wk=1, st=7)),   # 16 wavefronts, direct to LDS
+    (128, 2048, 256, dict(wm=2, rm=4, wn=1, rn=4, mf=16, bk=128, sk=2, wk=1, st=8)),   # written-out order: no barrier ends its last tile
+    (256, 1024, 128, dict(wm=1, rm=4, wn=1, rn=4, mf=32, bk=64, sk=2, wk=1, st=1)),    # 256 accumulators, one buffer: the sum area exceeds the tiles
+])
+def test_gemm_int8_k_divisions(oracle, M, K, N, kn):
+    """The reduce split of the int8 operator: across workgroups (exact whatever the order of the
+    atomic adds) and across wavefront groups; twice through one plan, the second launch over the
+    first one's result (the zero fill is part of the plan)."""
+    _gemm_int8_case(oracle, M, K, N, kn, None)
+    key = key_of("gemm", "gemm_int8", (M, K, N))
+    _, bufs = TASK_TABLE[key].func(M, K, N)
+    a, b = seeded_inputs(bufs, seed=K + 1)
+    g = None
+    if kn.get("st") in (6, 7, 8):
+        g = {k: [] for k in KEYS}
+        g["inline"], g["special"] = [[0]], [[-1, 0], [0]]
+    s, _ = schedule_with_config(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], g))
+    func = build(s, bufs, "rocm")
+    ins = [torch.from_numpy(x).cuda() for x in (a, b)]
+    out = torch.full((M, N), -77, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        func(*ins, out)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), oracle.gemm_i8_c(a, b))
+    func.close()
+    # stores that write finished sums do not combine with a divided K
+    if kn.get("st") == 7 and kn["bk"] == 2 * (32 if kn["mf"] == 32 else 64):
+        with pytest.raises(InvalidConfig):
+            g2 = {k: [] for k in KEYS}
+            g2["inline"], g2["special"] = [[0]], [[-1, 0], [4]]
+            schedule_with_config(key, Config([gcfg(M, N, ceil_div(K, 64) * 64, **kn)], g2))
+
+
 def _gemm_int8_case(oracle, M, K, N, kn, store):
     register(gemm_int8, "gemm", "gemm_int8", (M, K, N), "rocm", 0)
     key = key_of("gemm", "gemm_int8", (M, K, N))

@@ -121,10 +121,26 @@ def test_lowering_rejects_bad_configs():
     # split-K adds the zero-fill kernel and multiplies the grid
     s, _ = schedule_with_config(GEMM, Config([_gemm_cfg([16, 2, 1, 32], [16, 2, 1, 32], [2, 32, 16])], None))
     assert [x.kernel for x in s.specs] == ["fill_zero_f32", "igemm_f32"] and s.specs[1].grid[0] == 512
-    # int8 never splits K
+    # int8 the same (integer atomic adds), or wavefront groups that add up in LDS
     i8 = _gemm_cfg([16, 2, 4, 32], [16, 2, 4, 32], [2, 32, 64])
-    with pytest.raises((gfx950.InvalidConfig, AssertionError)):
+    s, _ = schedule_with_config(I8, Config([i8], None))
+    assert [x.kernel for x in s.specs] == ["fill_zero_f32", "gemm_i8"] and s.specs[1].grid[0] == 512
+    assert s.specs[1].defines["SPLITK"] == 2 and "WAVES_K" not in s.specs[1].defines
+    i8["reorder"] = [[1, 1]]
+    with pytest.raises(gfx950.InvalidConfig):          # 256 accumulators x 256 lanes of the second group: 256 KiB
         schedule_with_config(I8, Config([i8], None))
+    i8 = _gemm_cfg([32, 2, 2, 32], [32, 2, 2, 32], [2, 32, 64])
+    i8["reorder"] = [[1, 1]]
+    s, _ = schedule_with_config(I8, Config([i8], None))
+    assert [x.kernel for x in s.specs] == ["gemm_i8"] and s.specs[0].grid[0] == 1024
+    assert s.specs[0].defines["WAVES_K"] == 2 and s.specs[0].block[0] == 2 * 2 * 2 * 64
+    # ... but finished-sum stores (early stores of the last tile) need an undivided K
+    g = _gemm_cfg(None, None, None)
+    g.update(spatial=[], reduce=[], unroll=[], fuse=[], reorder=[], inline=[[0]], special=[[-1, 0], [4]])
+    i8 = _gemm_cfg([16, 2, 4, 32], [16, 2, 4, 32], [2, 32, 64], stages=7)
+    schedule_with_config(I8, Config([_gemm_cfg([16, 2, 4, 32], [16, 2, 4, 32], [1, 64, 64], stages=7)], g))
+    with pytest.raises(gfx950.InvalidConfig):
+        schedule_with_config(I8, Config([i8], g))
 
 
 def test_k_streaming_lowering():

@@ -3,8 +3,8 @@
 The hand-picked cases of test_gpu_parity.py cover the knobs one by one; here
 points are drawn from the operators' own spaces (the same sub-spaces the search
 walks: tile splits, K splits, pipeline depths, traversal, K division, plus the
-task-level knobs and the graph-level inline flag), so that combinations nobody
-thought of are run too. Points the templates refuse on the host are redrawn,
+task-level knobs and the graph-level inline and merge flags), so that combinations
+nobody thought of are run too. Points the templates refuse on the host are redrawn,
 as the search does. The draw is seeded by the case, so the points are the same
 in every process (and can be compiled ahead of time without a device).
 
@@ -45,14 +45,16 @@ def test_random_point_vs_oracle(oracle, shape_index, point):
     if kind == "int8":
         assert np.array_equal(out, oracle.gemm_i8_c(host[0], host[1])), what
         return
-    if kind == "gemm":
-        ref = oracle.gemm_f32_c(host[0], host[1])
+    if kind in ("gemm", "gemm_tn", "gemm_tt", "gemm_nt"):
+        ref = oracle.gemm_f32_c(host[0], host[1], transA=kind[-2] == "t", transB=kind[-1] == "t")
     elif kind == "bgemm":
         ref = np.stack([oracle.gemm_f32_c(host[0][b], host[1][b]) for b in range(args[0])])
-    elif kind in ("conv", "gconv"):
+    elif kind in ("conv", "gconv", "convb"):
         ref = oracle.conv2d_nchw_c(host[0], host[1], args[6], args[7], args[8], args[9])
     else:
         ref = oracle.depthwise_nchw_c(host[0], host[1], args[6], args[7], args[8])
+    if kind in ("convb", "dwb"):
+        ref = oracle.bias_add_nchw_np(ref, host[2])
     ref = np.asarray(ref, np.float64)
     err = float(np.max(np.abs(out.astype(np.float64) - ref)) / np.max(np.abs(ref)))
     assert err <= TOL, (err,) + what

@@ -263,7 +263,7 @@ def test_depthwise_lane_shifts_run_with_every_lane_switched_on(special):
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
-@pytest.mark.parametrize("shape_index", [0, 3, 4, 7, 8, 11, 13, 14, 18, 20])
+@pytest.mark.parametrize("shape_index", [0, 3, 4, 7, 8, 11, 13, 14, 18, 20, 22, 25, 27, 29])
 def test_random_points_of_the_spaces_pass_the_static_checks(shape_index):
     """The generated assembly of points drawn at random from the schedule spaces (the same points
     the device parity test runs): no accumulator read before the matrix core has written it, no

@@ -761,6 +761,9 @@ def schedule(task_key, slevel=4, rlevel=3, op_trial=50, graph_trial=10, op_stop=
             op_config = op_scheduler.schedule(configs, method=method, use_model=use_model,
                                               perf_path=perf_path)
             configs.op_config_lst.append(op_config)
+            # its compile workers go before the next scheduler starts its own: the workers load the
+            # HIP runtime, and a machine may bound the number of processes that do
+            op_scheduler.close()
 
         if verbose:
             print("space size", total_size)

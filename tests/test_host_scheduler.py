@@ -379,6 +379,23 @@ def test_schedule_random_method_and_conv_graph():
     assert 1 in calls and None in calls
 
 
+def test_an_operator_schedulers_workers_are_closed_before_the_next_scheduler_starts(monkeypatch):
+    """Compile workers load the HIP runtime; two pools alive at once doubled the number of
+    processes holding the device (a machine may bound it)."""
+    import flextensor_amd.scheduler as sch
+    events = []
+    real_close, real_init = sch.OpScheduler.close, sch.GraphScheduler.__init__
+    monkeypatch.setattr(sch.OpScheduler, "close", lambda self: (events.append("op closed"), real_close(self))[1])
+
+    def init(self, *a, **k):
+        events.append("graph scheduler")
+        real_init(self, *a, **k)
+    monkeypatch.setattr(sch.GraphScheduler, "__init__", init)
+    schedule(CONV, op_trial=2, graph_trial=1, parallel=2, method="random",
+             evaluator=lambda k, c, p, n: 1.0, verbose=False)
+    assert events.index("op closed") < events.index("graph scheduler")
+
+
 def test_failing_candidates_become_inf_and_search_survives():
     np.random.seed(2)
     n = {"calls": 0}

@@ -10,7 +10,7 @@ the static check of the kernels' assembly (isa_check).
 import os
 import sys
 
-from ..measure import get_measurer
+from ..measure import WrongResult, get_measurer
 from ..scheduler import schedule_with_config
 from ..task import TASK_TABLE
 
@@ -34,13 +34,11 @@ def test(task_key, configs, dev_id=None, rpc_info=None, check_result=False):
     dev_id = dev_id if dev_id is not None else task.dev_id
     time_cost = evaluate(task_key, s, bufs, task.target, dev_id, 100, rpc_info)
     if check_result:
-        m = get_measurer(task_key)
-        built = s.build()
-        built(*m.sets[0])
-        ok, metric = m.check(m.sets[0][-1])
-        built.close()
-        print("Test correctness...", "passed!" if ok else "failed!", "metric", metric)
-        # and the assembly: no read of an MFMA's result before the matrix core has written it
+        # against the default-schedule kernels on the device, then the static checks of the assembly
+        try:
+            print("Test correctness...", "passed!", "metric", s.verify(static=False))
+        except WrongResult as e:
+            print("Test correctness...", "failed!", e)
         from .. import isa_check
         if os.path.exists(isa_check.HIPCC):
             early = isa_check.check_plan(s)

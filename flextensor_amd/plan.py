@@ -37,6 +37,31 @@ class KernelPlan(object):
     def build(self, static_workspace=False):
         return BuiltPlan(self, static_workspace=static_workspace)
 
+    def verify(self, static=True):
+        """Run the plan once on the task's seeded inputs and compare the result with the
+        default-schedule kernels on the device (the gate every candidate of a search passes):
+        fp32 max|out - ref| / max|ref| <= 1e-5, int32 bit-exact. With ``static`` and hipcc
+        installed the generated assembly goes through the static checks as well. Returns the
+        metric; raises measure.WrongResult otherwise. For plans that did not come out of a
+        search: a config replayed from a log, or written by hand."""
+        import os
+        from . import isa_check
+        from .measure import WrongResult, get_measurer
+        m = get_measurer(self.task_key)
+        built = self.build()
+        try:
+            built(*m.sets[0])
+            ok, metric = m.check(m.sets[0][-1])
+        finally:
+            built.close()
+        if not ok:
+            raise WrongResult("%s: result differs from the default schedule's (metric %g)" % (self.task_key, metric))
+        if static and os.path.exists(isa_check.HIPCC):
+            found = isa_check.check_plan(self)
+            if found:
+                raise WrongResult("%s: static check of the assembly: %s" % (self.task_key, found[:2]))
+        return metric
+
     def with_clock_probe(self):
         """A copy of the plan whose main kernel is the instrumented build of its template
         (FT_CLKPROBE): every workgroup writes the shader clocks and the ticks of the 100 MHz

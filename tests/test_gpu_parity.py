@@ -1431,6 +1431,27 @@ def test_correctness_gate_rejects_wrong_output():
     assert compare_on_device(bad, m.sets[0][-1], current_stream())[0] is False
 
 
+def test_plan_verify_runs_the_gate_and_the_static_checks():
+    """KernelPlan.verify(): what a replayed or hand-written config is checked with (the candidates of
+    a search pass the same gate inside the measurer)."""
+    import flextensor_amd.measure as measure
+    for key in ("gemm_gemm_(256, 256, 256)_rocm(0)", "conv2d_baseline0_(1, 64, 56, 56, 64, 3, 1, 1, 1, 1)_rocm(0)",
+                "gemm_gemm_int8_(4096, 4096, 4096)_rocm(0)"):
+        s, _ = schedule_with_config(key, Config([], None))
+        assert s.verify() <= TOL
+    key = "gemm_gemm_(256, 256, 256)_rocm(0)"
+    s, _ = schedule_with_config(key, Config([], None))
+    m = measure.get_measurer(key)
+    keep = m.ref.clone()
+    m.ref += 1.0                                   # corrupt the default-schedule result
+    try:
+        with pytest.raises(WrongResult):
+            s.verify(static=False)
+    finally:
+        m.ref.copy_(keep)
+    assert s.verify(static=False) <= TOL
+
+
 def test_builtplan_rejects_mismatched_tensors():
     key = "gemm_gemm_(256, 256, 256)_rocm(0)"
     s, bufs = schedule_with_config(key, Config([], None))

@@ -131,3 +131,7 @@ baseline_conv_shapes = [
 ]
 baseline_depthwise_shapes = [(8, 512, 28, 28, 1, 3, 3, 1, 1, 1)]
 baseline_gemm_int8_shapes = [(4096, 4096, 4096)]
+# further int8 GEMMs (M, K, N): smaller cubes and two products with few tiles and a long K,
+# where the reduce split decides (across workgroups or across wavefront groups)
+gemm_int8_shapes = [(512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048),
+                    (1024, 4096, 1024), (512, 8192, 512)]

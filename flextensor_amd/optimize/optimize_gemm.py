@@ -6,12 +6,13 @@ flextensor/optimize/optimize_gemm.py:18-116 for the gfx950 backend.
 """
 import argparse
 
-from ..configs.shapes import baseline_gemm_shapes, baseline_gemm_int8_shapes, gemm_shapes
+from ..configs.shapes import baseline_gemm_shapes, baseline_gemm_int8_shapes, gemm_int8_shapes, gemm_shapes
 from ..task import Task
 from .common import init_arg_parser, run_driver
 
 SHAPES = {"baseline": [("gemm", s) for s in baseline_gemm_shapes],
           "int8": [("gemm_int8", s) for s in baseline_gemm_int8_shapes],
+          "int8_more": [("gemm_int8", s) for s in gemm_int8_shapes],
           "pow2": [("gemm", tuple(s)) for s in gemm_shapes]}
 
 

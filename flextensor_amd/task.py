@@ -14,7 +14,7 @@ from .te import placeholder
 from .configs.shapes import (gemm_shapes, yolo_shapes, yolo_shapes_b8, grouped_shapes, dilation_shapes,
                              depthwise_shapes, depthwise_shapes_b8, depthwise_shapes_b16,
                              baseline_conv_shapes, baseline_depthwise_shapes, baseline_gemm_shapes,
-                             baseline_gemm_int8_shapes, google_shapes, res_shapes, squeeze_shapes,
+                             baseline_gemm_int8_shapes, gemm_int8_shapes, google_shapes, res_shapes, squeeze_shapes,
                              vgg_16_shapes, test_conv_shapes, mobilev2_shapes, overfeat_shapes)
 
 # table name -> conv2d shapes, the names of flextensor/task.py:274-284 plus this backend's benchmark shapes
@@ -143,7 +143,7 @@ def _register_all():
         for shape in gemm_shapes + baseline_gemm_shapes:
             N, K, M = shape
             register(gemm, "gemm", "gemm", (N, K, M), ROCM_TARGET, j)
-        for shape in baseline_gemm_int8_shapes:
+        for shape in baseline_gemm_int8_shapes + gemm_int8_shapes:
             N, K, M = shape
             register(gemm_int8, "gemm", "gemm_int8", (N, K, M), ROCM_TARGET, j)
         for name, shapes in conv2d_shape_dict.items():

@@ -103,6 +103,11 @@ def roofline(name, bound, dtype, ops, nbytes, ms, plan, clock=None):
         out["shader_clock_ghz"] = clock["ghz"]
         out["shader_clock_ghz_p5_p95"] = [clock["ghz_min"], clock["ghz_max"]]
         out["workgroup_life_ms"] = clock["workgroup_us"] * 1e-3
+        if "time_axis_us" in clock:
+            # microseconds after a launch's first workgroup began: last begin, first and last end of a
+            # workgroup (its first wavefront's stores completed); gap = last end -> first begin of the
+            # next launch; period = begin to begin
+            out["time_axis_us"] = clock["time_axis_us"]
         if bound == "mfma":
             # the same fraction against the peak at the clock the part sustains under this load
             out["frac_at_sustained_clock"] = out["frac"] * NOMINAL_GHZ / clock["ghz"]
@@ -110,8 +115,16 @@ def roofline(name, bound, dtype, ops, nbytes, ms, plan, clock=None):
 
 
 def shader_clock(m, plan):
+    """The sustained clock and, on one time axis of the device's 100 MHz counter, where a launch's
+    time goes when launches follow one another (Measurer.time_axis): both read inside instrumented
+    builds of the same kernel, after the timing."""
     try:
-        return m.shader_clock(plan, ms=TIMED_WINDOW_MS, warm_ms=WARM_MS)
+        clock = m.shader_clock(plan, ms=TIMED_WINDOW_MS, warm_ms=WARM_MS)
+        if clock is not None:
+            axis = m.time_axis(plan, launches=max(int(TIMED_WINDOW_MS / max(clock["workgroup_us"] * 1e-3, 2e-3)), 200),
+                               warm_ms=WARM_MS)
+            clock["time_axis_us"] = {k: axis[k] for k in ("period", "start_skew", "first_end", "last_end", "gap")}
+        return clock
     except Exception as e:  # noqa: BLE001 - the clock is an annotation, the timing stands without it
         print("shader clock probe failed: %s" % e, file=sys.stderr)
         return None

@@ -256,6 +256,47 @@ class Measurer(object):
                 "ghz_max": float(np.percentile(ghz, 95)), "workgroup_us": float(np.median(clk[:, 1]) / 100.0),
                 "workgroups": int(len(clk))}
 
+    def time_axis(self, plan, launches=3000, warm_ms=150.0):
+        """Where the time of a launch goes when launches follow one another on one stream, read
+        inside the kernels: two instrumented builds of ``plan`` (KernelPlan.with_clock_probe with
+        ``absolute=True``) are launched in turn, so the stamps of the last two launches survive,
+        and every workgroup reports the device's 100 MHz counter at its begin and at the
+        completion of its first wavefront's stores. Returns microseconds: ``period`` (first begin
+        of one launch to first begin of the next), ``start_skew`` (first to last begin of a launch),
+        ``first_end`` / ``last_end`` (after the launch's first begin) and ``gap`` (last end of one
+        launch to first begin of the next: the other wavefronts' last stores, the write-back of
+        what the launch left in the caches, and the dispatch of the next launch). 10 ns steps."""
+        import torch
+        builds = [plan.with_clock_probe(absolute=True).build() for _ in range(2)]
+        try:
+            sets = self.sets
+            for b in builds:
+                b(*sets[0])
+            torch.cuda.synchronize()
+            for b in builds:
+                ok, metric = self.check(sets[0][-1])
+                if not ok:
+                    raise WrongResult("instrumented build differs from the default schedule (metric %g)" % metric)
+            builds[0].time(sets, warmup=1, iters=5, warm_ms=warm_ms)
+            # one call enqueues the whole alternating sequence, so the launches follow one another
+            # as closely as the device lets them (launched one by one the host would set the pace)
+            per = [[x.launches(ts) for ts in sets] for x in builds]
+            pairs = max(int(launches) // 2, 1)      # an even number: the second build launches last
+            seq = [d for i in range(2 * pairs) for d in per[i % 2][i % len(sets)]]
+            rt._check(rt.lib().ftr_launch_seq(rt._desc_array(seq), len(seq), ctypes.c_void_p(current_stream())),
+                      "ftr_launch_seq")
+            torch.cuda.synchronize()
+            a, b = [x.scratch["clk_probe"].cpu().numpy().astype(np.int64) for x in builds]
+        finally:
+            for x in builds:
+                x.close()
+        a, b = a[a[:, 1] - a[:, 0] >= 20], b[b[:, 1] - b[:, 0] >= 20]     # workgroups that found work
+        t0 = a[:, 0].min()
+        us = lambda ticks: float(ticks) / 100.0
+        return {"period": us(b[:, 0].min() - t0), "start_skew": us(a[:, 0].max() - t0),
+                "first_end": us(a[:, 1].min() - t0), "last_end": us(a[:, 1].max() - t0),
+                "gap": us(b[:, 0].min() - a[:, 1].max()), "workgroups": int(len(a))}
+
     def evaluate(self, plan, number=10, warmup=2, warm_ms=WARM_MS, timeout=0.0):
         """ms per run of ``plan``; raises on build failure or wrong output.
         Candidates are compiled between measurements, so each one meets an

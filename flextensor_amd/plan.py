@@ -62,18 +62,21 @@ class KernelPlan(object):
                 raise WrongResult("%s: static check of the assembly: %s" % (self.task_key, found[:2]))
         return metric
 
-    def with_clock_probe(self):
+    def with_clock_probe(self, absolute=False):
         """A copy of the plan whose main kernel is the instrumented build of its template
         (FT_CLKPROBE): every workgroup writes the shader clocks and the ticks of the 100 MHz
         counter it lived into the workspace ``clk_probe`` ([workgroups][2] int64). Same work,
-        same launch geometry; used to read the clock the kernel sustains, never timed."""
+        same launch geometry; used to read the clock the kernel sustains, never timed.
+        ``absolute``: the two numbers are the 100 MHz counter's own readings at the workgroup's
+        begin and end instead (one counter for the whole device), which puts the workgroups of
+        several launches on one time axis."""
         import copy
         idx = [i for i, s in enumerate(self.specs) if s.template in PROBE_TEMPLATES]
         if not idx:
             raise ValueError("no kernel of this plan can carry the clock probe")
         specs = list(self.specs)
         spec = copy.copy(specs[idx[-1]])
-        spec.defines = dict(spec.defines, CLKPROBE=1)
+        spec.defines = dict(spec.defines, CLKPROBE=2 if absolute else 1)
         spec.args = list(spec.args) + [("buf", "clk_probe")]
         nwg = spec.grid[0] * spec.grid[1] * spec.grid[2]
         spec.workspace = dict(spec.workspace, clk_probe=((nwg, 2), "int64"))

@@ -437,10 +437,18 @@ static __device__ __forceinline__ f32x4 ld_f32x4(__amdgpu_buffer_rsrc_t r, unsig
  * completion of its first wavefront's last store. */
 #ifdef FT_CLKPROBE
 #define CLK_PARAM , unsigned long long* __restrict__ ft_clk
+#if FT_CLKPROBE == 2
+/* the two stamps of the 100 MHz counter themselves (it is common to the device): when the workgroup began and
+ * when its first wavefront's stores had completed, to lay the workgroups of consecutive launches on one time axis */
+#define CLK_BEGIN const unsigned long long ft_r0 = wall_clock64();
+#define CLK_END do { __builtin_amdgcn_s_waitcnt(0x0F70); \
+        if (threadIdx.x == 0) { ft_clk[2 * blockIdx.x] = ft_r0; ft_clk[2 * blockIdx.x + 1] = wall_clock64(); } } while (0)
+#else
 #define CLK_BEGIN const unsigned long long ft_t0 = __builtin_readcyclecounter(), ft_r0 = wall_clock64();
 #define CLK_END do { __builtin_amdgcn_s_waitcnt(0x0F70); \
         if (threadIdx.x == 0) { ft_clk[2 * blockIdx.x] = __builtin_readcyclecounter() - ft_t0; \
                                 ft_clk[2 * blockIdx.x + 1] = wall_clock64() - ft_r0; } } while (0)
+#endif
 #else
 #define CLK_PARAM
 #define CLK_BEGIN

@@ -131,9 +131,17 @@ def test_shader_clock_is_read_inside_the_kernels():
         assert [(k.kernel, dict(k.defines), list(k.args)) for k in s.specs] == before
         assert probe.specs[-1].defines["CLKPROBE"] == 1 and probe.specs[-1].args[-1] == ("buf", "clk_probe")
         assert "clk_probe" in probe.workspaces and "clk_probe" not in s.workspaces
-        clk = Measurer(key, seed=4).shader_clock(s, ms=3.0, warm_ms=30.0)
+        m = Measurer(key, seed=4)
+        clk = m.shader_clock(s, ms=3.0, warm_ms=30.0)
         assert clk is not None and 0.5 < clk["ghz"] < 2.6 and clk["ghz_min"] <= clk["ghz"] <= clk["ghz_max"]
         assert 0.2 < clk["workgroup_us"] < 1000 and clk["workgroups"] >= 1
+        # the same with the counter's own readings: two launches on one time axis
+        assert s.with_clock_probe(absolute=True).specs[-1].defines["CLKPROBE"] == 2
+        axis = m.time_axis(s, launches=201, warm_ms=30.0)        # odd: rounded down to whole pairs
+        assert 0 <= axis["start_skew"] < axis["first_end"] <= axis["last_end"] < axis["period"] < 1000
+        assert abs(axis["gap"] - (axis["period"] - axis["last_end"])) < 1e-6 and axis["gap"] > 0
+        per_launch = m.evaluate(s, number=200, warm_ms=30.0) * 1e3
+        assert 0.5 * per_launch < axis["period"] < 2.0 * per_launch + 2.0
 
 
 def test_time_limit_abandons_an_overrunning_measurement_and_recovers():

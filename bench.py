@@ -311,8 +311,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--only-headline", action="store_true", help="skip the per_config table")
     ap.add_argument("--no-clock", action="store_true",
-                    help="skip the in-kernel shader clock probe (an instrumented build of the same kernel, "
-                         "run after the timing; under a profiler it would show up as extra dispatches)")
+                    help="skip the in-kernel probes of the shader clock and of the launches' time axis "
+                         "(instrumented builds of the same kernel, run after the timing; under a profiler "
+                         "they would show up as extra dispatches)")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="instead of a workload, run a plain device copy of this many MiB "
                          "(bandwidth yardstick; calibrates FETCH_SIZE/WRITE_SIZE)")

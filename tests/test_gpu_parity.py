@@ -138,7 +138,8 @@ def test_shader_clock_is_read_inside_the_kernels():
         # the same with the counter's own readings: two launches on one time axis
         assert s.with_clock_probe(absolute=True).specs[-1].defines["CLKPROBE"] == 2
         axis = m.time_axis(s, launches=201, warm_ms=30.0)        # odd: rounded down to whole pairs
-        assert 0 <= axis["start_skew"] < axis["first_end"] <= axis["last_end"] < axis["period"] < 1000
+        # (a grid larger than what the device holds at once may begin its last workgroup after its first has ended)
+        assert 0 <= axis["start_skew"] <= axis["last_end"] and 0 < axis["first_end"] <= axis["last_end"] < axis["period"] < 1000
         assert abs(axis["gap"] - (axis["period"] - axis["last_end"])) < 1e-6 and axis["gap"] > 0
         per_launch = m.evaluate(s, number=200, warm_ms=30.0) * 1e3
         assert 0.5 * per_launch < axis["period"] < 2.0 * per_launch + 2.0

@@ -128,3 +128,30 @@ def test_perf_path_is_written_by_the_driver(capsys, tmp_path):
     common.run_driver(args, shapes, optimize_gemm.make_task, "gemm")
     capsys.readouterr()
     assert os.path.isdir(perf) and os.listdir(perf)
+
+
+def test_polish_refines_a_log_one_knob_at_a_time(oracle, tmp_path, capsys):
+    """flextensor_amd.optimize.polish: every line of the log comes out (refined or as it was),
+    still a key:json line the reference's reader takes, still correct against the oracle; a line
+    of a task that is not registered is copied."""
+    from flextensor_amd.optimize import polish
+    from flextensor_amd.templates.gfx950 import default_config
+    key = "gemm_gemm_(256, 256, 256)_rocm(0)"
+    ops, _ = TASK_TABLE[key].func(*TASK_TABLE[key].args)
+    cfg = Config([default_config(ops[0])], {k: [] for k in default_config(ops[0])})
+    foreign = "gemm_gemm_(3, 5, 7)_cuda(0):" + json.dumps(cfg)
+    src, dst = tmp_path / "in.log", tmp_path / "out.log"
+    src.write_text(key + ":" + json.dumps(cfg) + "\n" + foreign + "\n")
+    assert polish.main(["--log", str(src), "--out", str(dst), "--number", "60", "--threshold", "0.03"]) == 0
+    said = capsys.readouterr().out
+    assert "entries refined" in said and key in said
+    entries = read_log(str(dst))
+    assert [k for k, _ in entries] == [key, "gemm_gemm_(3, 5, 7)_cuda(0)"]
+    assert dst.read_text().split("\n")[1] == foreign
+    host, out = replay_output(key, entries[0][1], seed=11)
+    assert rel(out, oracle.gemm_f32_c(host[0], host[1])) <= TOL
+    # the neighbours differ from the entry in exactly one knob
+    for what, cand in polish.neighbours(key, entries[0][1]):
+        a, b = json.loads(json.dumps(entries[0][1])), json.loads(json.dumps(cand))
+        diff = [k for k in a[0][0] if a[0][0][k] != b[0][0][k]] + [k for k in a[1] if a[1].get(k) != b[1].get(k)]
+        assert len(diff) == 1, (what, diff)

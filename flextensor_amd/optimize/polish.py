@@ -5,12 +5,16 @@
 A search ends at a point of a large space after a bounded number of trials; kernels change
 afterwards (a cheaper set-up shifts the balance between LDS layouts, for one). This pass takes
 every ``key:json`` line of a log, measures it, and tries the neighbours along the knobs that
-cost nothing to enumerate: the LDS layout (`lds_pad`), the number of k blocks the next tile's
-loads are spread over (depth 8), the traversal group height and the XCD renumbering. A
-neighbour replaces the entry when it is faster by more than ``--threshold`` (default 1.2 %)
-in two measurements and again in a second pair against the then-current entry; every
-measurement passes the on-device correctness gate. Lines of tasks that are not registered, or
-whose last kernel is not the fp32 contraction template, are copied as they are.
+cost nothing to enumerate: the task's enumerated knobs (the LDS layout `lds_pad`, the int8 store
+forms, the depthwise variants), the number of k blocks the next tile's loads are spread over
+(depth 8), the traversal group height and the XCD renumbering, for depthwise the wavefronts per
+workgroup. A
+neighbour replaces the entry when it is faster by more than ``--threshold`` (default 1 %) in a
+first measurement and then in every one of four rounds that alternate between it and the
+then-current entry (kernels near the launch floor time bimodally; a single pair of
+measurements lets noise through); every
+measurement passes the on-device correctness gate. Lines of tasks that are not registered are
+copied as they are.
 """
 import argparse
 import json
@@ -23,6 +27,9 @@ from ..templates import gfx950
 from ..utils import Config
 
 
+ROUNDS = 4          # alternating confirmations a neighbour has to win, all of them
+
+
 def _time(measurer, plan, number):
     return min(measurer.evaluate(plan, number=number) for _ in range(2))
 
@@ -31,22 +38,30 @@ def neighbours(key, cfg):
     """[(what, Config)] one knob away from ``cfg``."""
     out = []
     task = TASK_TABLE[key]
+    # the task's enumerated knobs (LDS layout, store forms, the depthwise variants): every other value
     names = list(task.special_space)
-    if "lds_pad" in names:
-        at = names.index("lds_pad")
-        special = [list(x) for x in (cfg.graph_config.get("special") or [])]
-        while len(special) <= at:
-            special.append(list(gfx950.SPECIAL_DEFAULTS[names[len(special)]]))
-        for pad in task.special_space["lds_pad"].static_entities:
-            if list(pad) != special[at]:
+    special = [list(x) for x in (cfg.graph_config.get("special") or [])]
+    while len(special) < len(names):
+        special.append(list(gfx950.SPECIAL_DEFAULTS[names[len(special)]]))
+    for at, name in enumerate(names):
+        for value in task.special_space[name].static_entities:
+            if list(value) != special[at]:
                 s2 = [list(x) for x in special]
-                s2[at] = list(pad)
-                out.append(("lds_pad %s" % list(pad), Config(cfg.op_config_lst, dict(cfg.graph_config, special=s2))))
+                s2[at] = list(value)
+                out.append(("%s %s" % (name, list(value)), Config(cfg.op_config_lst, dict(cfg.graph_config, special=s2))))
     pos = [i for i, c in enumerate(cfg.op_config_lst) if c.get("spatial")]
     if not pos:
         return out
     pos = pos[0]
     op = cfg.op_config_lst[pos]
+    if len(op["spatial"]) == 4:          # depthwise: wavefronts per workgroup
+        waves = (op.get("fuse") or [[4]])[0][0]
+        for x in (1, 2, 4, 8):
+            if x != waves:
+                ops = [dict(c) for c in cfg.op_config_lst]
+                ops[pos]["fuse"] = [[x]]
+                out.append(("wavefronts %d" % x, Config(ops, dict(cfg.graph_config))))
+        return out
 
     def with_op(knob, value):
         ops = [dict(c) for c in cfg.op_config_lst]
@@ -63,10 +78,10 @@ def neighbours(key, cfg):
     return out
 
 
-def polish_entry(key, cfg, threshold=0.012, number=400, longest_ms=0.2):
+def polish_entry(key, cfg, threshold=0.01, number=1000, longest_ms=0.2):
     """(Config, ms before, ms after, [accepted moves]); the entry itself when nothing is faster."""
     plan, _ = schedule_with_config(key, cfg)
-    if plan.specs[-1].kernel != "igemm_f32":
+    if plan.specs[-1].kernel not in ("igemm_f32", "gemm_i8", "depthwise_f32"):
         return cfg, None, None, []
     m = get_measurer(key)
     base = _time(m, plan, number)
@@ -88,10 +103,12 @@ def polish_entry(key, cfg, threshold=0.012, number=400, longest_ms=0.2):
             except Exception:  # noqa: BLE001  (refused on the host, failed to build, wrong result)
                 continue
             if t < best * (1.0 - threshold):
-                again_best = min(_time(m, schedule_with_config(key, best_cfg)[0], number), best)
-                again = min(_time(m, p1, number), t)
-                if again < again_best * (1.0 - threshold):
-                    best_cfg, best, improved = cand, again, True
+                # kernels near the launch floor time bimodally from one build to the next: the candidate
+                # has to win every one of several rounds that alternate with the current entry
+                p0, _ = schedule_with_config(key, best_cfg)
+                rounds = [(m.evaluate(p0, number=number), m.evaluate(p1, number=number)) for _ in range(ROUNDS)]
+                if all(c < b * (1.0 - threshold) for b, c in rounds):
+                    best_cfg, best, improved = cand, min(c for _, c in rounds), True
                     moves.append(what)
     return best_cfg, base, best, moves
 
@@ -100,8 +117,8 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--log", required=True, help="key:json lines to refine")
     ap.add_argument("--out", required=True, help="where the refined lines go (every line of --log, refined or not)")
-    ap.add_argument("--threshold", type=float, default=0.012)
-    ap.add_argument("--number", type=int, default=400, help="launches per timing")
+    ap.add_argument("--threshold", type=float, default=0.01)
+    ap.add_argument("--number", type=int, default=1000, help="launches per timing")
     ap.add_argument("-f", "--from_", type=int, default=0)
     ap.add_argument("-t", "--to", type=int, default=-1)
     args = ap.parse_args(argv)
